@@ -1,0 +1,170 @@
+/*
+ * lbtree -- C ABI of the MI355X (gfx950) tree-learner path.
+ *
+ * These entry points are what a Legate GPU task variant binds instead of the
+ * CUDA bodies of rapidsai/legate-boost's tree tasks. All pointers named
+ * "device" are plain HIP device pointers (for Legate: accessor.ptr() of a
+ * dense, C-ordered instance); `stream` is a hipStream_t passed as void*
+ * (context.get_task_stream()). No call keeps a pointer after it returns.
+ *
+ * Every function returns LBT_OK (0) or a negative status; the message for the
+ * last failure on the calling thread is available from lbt_last_error().
+ * The reference throws C++ exceptions at the same places
+ * (src/cpp_utils/cpp_utils.h:85-96 EXPECT, cpp_utils.cuh:45-58 CHECK_CUDA);
+ * the task glue turns a non-zero status into std::runtime_error.
+ */
+#ifndef LBTREE_H
+#define LBTREE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LBT_OK 0
+#define LBT_ERR_INVALID (-1)     /* bad argument (shape, dtype, null pointer, range) */
+#define LBT_ERR_HIP (-2)         /* a HIP runtime call failed */
+#define LBT_ERR_WORKSPACE (-3)   /* workspace missing or too small */
+#define LBT_ERR_UNSUPPORTED (-4) /* input outside what the kernels handle exactly */
+
+/* dtype of X; the reference dispatches on the same two types
+ * (src/cpp_utils/cpp_utils.h:177-182 type_dispatch_float). */
+#define LBT_F32 0
+#define LBT_F64 1
+
+/* Upper limit on split_samples, as in legateboost/models/tree.py:75-76. */
+#define LBT_MAX_SPLIT_SAMPLES 2048
+
+const char* lbt_last_error(void);
+int lbt_version(void);
+
+/* The eight task scalars of BUILD_TREE in their reference order
+ * (legateboost/models/tree.py:121-129, build_tree.cu:1292-1299), plus the
+ * histogram-cache budget that the reference hard-codes to 1e9 bytes
+ * (build_tree.cu:1004). hist_cache_bytes == 0 selects that constant. */
+typedef struct lbt_build_params {
+  int32_t max_depth;
+  int32_t max_nodes; /* must equal 2^(max_depth+1) - 1 */
+  int32_t split_samples;
+  int32_t seed;
+  int64_t dataset_rows;
+  double l1_regularization;
+  double l2_regularization;
+  double min_split_gain;
+  int64_t hist_cache_bytes;
+} lbt_build_params;
+
+/* Optional observation points of lbt_build_tree, for parity tests and
+ * profiling. Pointer members are DEVICE pointers unless marked host; any of
+ * them may be NULL. They have no counterpart in the reference. */
+typedef struct lbt_build_taps {
+  void* proposals;              /* X dtype [n_features*split_samples]; first n_bins valid */
+  int32_t* row_pointers;        /* [n_features+1] */
+  int32_t* quantised;           /* [n_rows*n_outputs*2] int32 (grad, hess) */
+  int64_t* node_sums;           /* [max_nodes*n_outputs*2] */
+  int32_t* positions;           /* [n_rows*2] (node,row) after the last update */
+  int32_t* positions_per_level; /* [max_depth*n_rows*2]; slot d = order used at depth d */
+  int64_t* histogram;           /* [nodes][n_outputs][n_bins][2] of the last histogram buffer */
+  int64_t histogram_capacity;   /* in: int64 elements available at `histogram` */
+  /* host outputs */
+  int32_t n_bins;
+  int32_t hist_node_begin;
+  int32_t hist_node_end;
+  double scales[4];             /* scale.grad, scale.hess, 1/scale.grad, 1/scale.hess */
+  int64_t* level_instances;       /* host [max_depth]: rows in all batches of the level */
+  int64_t* level_built_instances; /* host [max_depth]: rows of nodes whose histogram is built */
+  int32_t* level_built_nodes;     /* host [max_depth] */
+} lbt_build_taps;
+
+/* Bytes of device scratch lbt_build_tree needs for these shapes (an upper
+ * bound that does not depend on the data). Replaces the task-scoped
+ * legate::create_buffer allocations of build_tree.cu (:790-794, :880-933,
+ * :997, :1012, :1052, :1064). Returns 0 for invalid arguments. */
+size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_t n_outputs,
+                                      int32_t max_depth, int32_t split_samples, int32_t x_dtype,
+                                      int64_t hist_cache_bytes);
+
+/*
+ * BuildTreeTask::gpu_variant (src/models/tree/build_tree.cu:1274-1365).
+ *   X        device [n_rows][n_features], row-major, dtype x_dtype; holds global
+ *            rows [row_offset, row_offset+n_rows) (X_shape.lo[0])
+ *   g, h     device double [n_rows][n_outputs]
+ *   feature_set  device bytes [n_features] (non-zero = feature usable) or NULL
+ *                (optional 4th task input, build_tree.cu:1302-1307)
+ *   leaf, feature, split, gain, hessian  device outputs 0..4
+ *            ([max_nodes][n_outputs] f64, [max_nodes] i32, [max_nodes] f64,
+ *             [max_nodes] f64, [max_nodes][n_outputs] f64)
+ *   workspace    device scratch of at least lbt_build_tree_workspace_bytes(...)
+ * The call returns after the stream has been synchronised, like the
+ * reference (build_tree.cu:1356).
+ */
+int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
+                   int64_t n_rows, int32_t n_features, const double* g, const double* h,
+                   int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
+                   double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
+                   void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
+
+/*
+ * PredictTask::gpu_variant (src/models/tree/predict.cu:26-91).
+ *   leaf/feature/split  HOST arrays of n_trees device pointers, in the order
+ *                       the trees appear as task inputs (tree.py:264-273)
+ *   tree_nodes          HOST array: number of nodes of each tree
+ *   out                 device double [n_rows][n_outputs]; overwritten
+ * Work is enqueued on `stream`; the call does not synchronise.
+ */
+int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                int32_t n_trees, const double* const* leaf, const int32_t* const* feature,
+                const double* const* split, const int32_t* tree_nodes, int32_t n_outputs,
+                double* out);
+
+/* Device scratch needed by lbt_update_tree. */
+size_t lbt_update_tree_workspace_bytes(int64_t n_rows, int32_t n_outputs, int32_t n_nodes);
+
+/*
+ * UpdateTreeTask (src/models/tree/update_tree.cc:36-122; CPU-only in the
+ * reference). Re-accumulates g,h over the fixed structure and recomputes the
+ * leaves. Sums are formed in double by atomics, so leaf values agree with the
+ * reference's sequential sums to rounding (not bit-exact).
+ */
+int lbt_update_tree(void* stream, const void* X, int32_t x_dtype, int64_t n_rows,
+                    int32_t n_features, const double* g, const double* h, int32_t n_outputs,
+                    const int32_t* feature, const double* split, int32_t n_nodes,
+                    double l1_regularization, double l2_regularization, double* leaf_out,
+                    double* hessian_out, void* workspace, size_t workspace_bytes);
+
+/* ---- profiling (no counterpart in the reference) -------------------------- */
+
+#define LBT_PROF_PROPOSALS 0
+#define LBT_PROF_QUANTISE 1
+#define LBT_PROF_HISTOGRAM 2
+#define LBT_PROF_SCAN 3
+#define LBT_PROF_SPLIT 4
+#define LBT_PROF_POSITIONS 5
+#define LBT_PROF_OTHER 6
+#define LBT_PROF_PREDICT 7
+#define LBT_PROF_CLASSES 8
+
+typedef struct lbt_profile {
+  /* per kernel class: launches timed, summed GPU time (ms, HIP events on the
+   * stream of the call), and algorithmic bytes moved */
+  int64_t launches[LBT_PROF_CLASSES];
+  double ms[LBT_PROF_CLASSES];
+  double bytes[LBT_PROF_CLASSES];
+  /* histogram kernel per tree level of the most recent lbt_build_tree */
+  int32_t n_levels;
+  double level_ms[64];
+  double level_bytes[64];
+} lbt_profile;
+
+/* When enabled, lbt_build_tree / lbt_predict bracket their kernels with HIP
+ * events (this adds host synchronisation). Counters accumulate until reset. */
+void lbt_profile_enable(int on);
+void lbt_profile_reset(void);
+void lbt_profile_get(lbt_profile* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

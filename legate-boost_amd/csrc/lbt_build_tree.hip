@@ -1,0 +1,1453 @@
+// BuildTreeTask for one MI355X: split-proposal gather, gradient quantisation,
+// per-level histograms (LDS-privatised, merged by 64-bit integer atomics),
+// prefix scan + sibling subtraction, split evaluation with the reference's
+// tie rule, and the stable row->node partition.
+//
+// Semantics follow rapidsai/legate-boost src/models/tree/build_tree.cu and
+// build_tree.h (cited per kernel); the decomposition into kernels is this
+// library's own and is written for gfx950 (64-wide waves, 160 KB LDS per CU).
+#include "lbt_internal.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <limits>
+
+namespace lbt {
+namespace {
+
+constexpr int kThreads = 256;
+
+// ---------------------------------------------------------------------------
+// small helpers
+// ---------------------------------------------------------------------------
+
+template <typename T>
+struct KeyOf;
+template <>
+struct KeyOf<float> {
+  using type = uint32_t;
+};
+template <>
+struct KeyOf<double> {
+  using type = uint64_t;
+};
+
+// Order-preserving map from IEEE bits to unsigned integers (-0.0 < +0.0).
+__device__ inline uint32_t to_key(float v)
+{
+  uint32_t u = __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ inline uint64_t to_key(double v)
+{
+  uint64_t u = static_cast<uint64_t>(__double_as_longlong(v));
+  return (u & 0x8000000000000000ULL) ? ~u : (u | 0x8000000000000000ULL);
+}
+__device__ inline float from_key(uint32_t k)
+{
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+__device__ inline double from_key(uint64_t k)
+{
+  uint64_t u = (k & 0x8000000000000000ULL) ? (k & 0x7fffffffffffffffULL) : ~k;
+  return __longlong_as_double(static_cast<long long>(u));
+}
+
+__device__ inline void atomic_add_i64(int64_t* p, int64_t v)
+{
+  atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(v));
+}
+
+struct HistView {
+  I64Pair* data;  // [node - node_begin][K][B]
+  int node_begin;
+  int node_end;
+  int K;
+  int B;
+  __device__ bool contains(int node) const { return node >= node_begin && node < node_end; }
+  __device__ I64Pair* at(int node, int k, int bin) const
+  {
+    return data + ((static_cast<int64_t>(node - node_begin) * K + k) * B + bin);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// tree initialisation / output (build_tree.cu:785-861)
+// ---------------------------------------------------------------------------
+
+__global__ void init_tree_kernel(double* leaf, int32_t* feature, double* split, double* gain,
+                                 I64Pair* node_sums, int64_t max_nodes, int K)
+{
+  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i < max_nodes * K) {
+    leaf[i]      = 0.0;
+    node_sums[i] = I64Pair{0, 0};
+  }
+  if (i < max_nodes) {
+    feature[i] = -1;
+    split[i]   = 0.0;
+    gain[i]    = 0.0;
+  }
+}
+
+__global__ void write_hessian_kernel(double* hessian, const I64Pair* node_sums, int64_t n,
+                                     const double* scales)
+{
+  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i < n) hessian[i] = static_cast<double>(node_sums[i].hess) * scales[3];
+}
+
+__global__ void zero_kernel(uint4* p, int64_t n16)
+{
+  int64_t i      = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------
+// split proposals (build_tree.cu:867-964)
+// ---------------------------------------------------------------------------
+
+// draft[f][i] = X[row_i][f] for the S sampled rows; row_i from a fresh
+// minstd engine advanced by i (build_tree.cu:882-898).
+template <typename T>
+__global__ void gather_samples_kernel(const T* X, int64_t row_offset, int64_t n_rows, int F,
+                                      int S, int32_t seed, int64_t dataset_rows, T* draft)
+{
+  int64_t idx = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (idx >= static_cast<int64_t>(F) * S) return;
+  int i        = static_cast<int>(idx / F);
+  int j        = static_cast<int>(idx % F);
+  uint32_t x   = minstd_seed(static_cast<uint32_t>(seed));
+  x            = minstd_discard(x, static_cast<uint64_t>(i));
+  x            = minstd_next(x);
+  double u     = uniform01(x);
+  double b     = static_cast<double>(dataset_rows - 1) + 1.0;
+  int64_t row  = static_cast<int64_t>((u * (b - 0.0)) + 0.0);
+  bool has     = row >= row_offset && row <= row_offset + n_rows - 1;
+  draft[static_cast<int64_t>(j) * S + i] = has ? X[(row - row_offset) * F + j] : T(0);
+}
+
+// One workgroup per feature: bitonic sort of the S samples in LDS on
+// order-preserving integer keys, then drop values equal to their predecessor
+// (thrust::sort + unique_copy, build_tree.cu:908-931).
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+  sort_unique_kernel(const T* draft, int S, int P, T* uniq, int32_t* counts)
+{
+  using Key = typename KeyOf<T>::type;
+  extern __shared__ unsigned char smem_raw[];
+  Key* keys       = reinterpret_cast<Key*>(smem_raw);
+  __shared__ int s_cnt[kThreads];
+  const int f     = blockIdx.x;
+  const T* src    = draft + static_cast<int64_t>(f) * S;
+  for (int i = threadIdx.x; i < P; i += kThreads) keys[i] = i < S ? to_key(src[i]) : ~Key(0);
+  __syncthreads();
+  for (int size = 2; size <= P; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = threadIdx.x; i < P / 2; i += kThreads) {
+        int lo      = 2 * i - (i & (stride - 1));  // index with the stride bit clear
+        int hi      = lo + stride;
+        bool up     = (lo & size) == 0;
+        Key a = keys[lo], b = keys[hi];
+        if ((a > b) == up) {
+          keys[lo] = b;
+          keys[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // thread t owns the contiguous slice [t*per, (t+1)*per)
+  const int per = (S + kThreads - 1) / kThreads;
+  int begin = threadIdx.x * per, end = min(S, begin + per);
+  int cnt = 0;
+  for (int i = begin; i < end; i++) {
+    bool keep = i == 0 || !(from_key(keys[i]) == from_key(keys[i - 1]));
+    cnt += keep ? 1 : 0;
+  }
+  s_cnt[threadIdx.x] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int t = 0; t < kThreads; t++) {
+      int c    = s_cnt[t];
+      s_cnt[t] = run;
+      run += c;
+    }
+    counts[f] = run;
+  }
+  __syncthreads();
+  int at = s_cnt[threadIdx.x];
+  T* dst = uniq + static_cast<int64_t>(f) * S;
+  for (int i = begin; i < end; i++) {
+    bool keep = i == 0 || !(from_key(keys[i]) == from_key(keys[i - 1]));
+    if (keep) dst[at++] = from_key(keys[i]);
+  }
+}
+
+// CSR row pointers (reduce_by_key + inclusive_scan, build_tree.cu:933-949)
+__global__ void row_pointers_kernel(const int32_t* counts, int F, int32_t* row_pointers)
+{
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    int run         = 0;
+    row_pointers[0] = 0;
+    for (int f = 0; f < F; f++) {
+      run += counts[f];
+      row_pointers[f + 1] = run;
+    }
+  }
+}
+
+// compact copy; the last proposal of each feature becomes +inf (build_tree.cu:953-956)
+template <typename T>
+__global__ void compact_proposals_kernel(const T* uniq, int S, const int32_t* row_pointers,
+                                         T* proposals, int32_t* bin_feature)
+{
+  const int f = blockIdx.x;
+  int b0 = row_pointers[f], b1 = row_pointers[f + 1];
+  for (int i = threadIdx.x; i < b1 - b0; i += blockDim.x) {
+    T v = uniq[static_cast<int64_t>(f) * S + i];
+    if (i == b1 - b0 - 1) v = std::numeric_limits<T>::infinity();
+    proposals[b0 + i]   = v;
+    bin_feature[b0 + i] = f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gradient quantiser (build_tree.cu:51-140, :168-204)
+// ---------------------------------------------------------------------------
+
+// One level of the fixed-order sum: chunk c covers 4096 entries; lane t adds
+// entries t, t+256, ... in order, then a binary tree (strides 128..1) joins the
+// 256 lanes. The reference leaves this order to thrust::reduce
+// (build_tree.cu:82-83); fixing it makes the two scale factors reproducible.
+template <bool kAbs>
+__global__ void __launch_bounds__(kThreads)
+  abs_sum_level_kernel(const double* a, const double* b, int64_t n, double* out_a, double* out_b)
+{
+  __shared__ double sa[kThreads];
+  __shared__ double sb[kThreads];
+  const int64_t c = blockIdx.x;
+  double xa = 0.0, xb = 0.0;
+  for (int j = 0; j < 16; j++) {
+    int64_t e = c * 4096 + threadIdx.x + static_cast<int64_t>(kThreads) * j;
+    if (e < n) {
+      xa += kAbs ? fabs(a[e]) : a[e];
+      xb += kAbs ? fabs(b[e]) : b[e];
+    }
+  }
+  sa[threadIdx.x] = xa;
+  sb[threadIdx.x] = xb;
+  __syncthreads();
+  for (int stride = kThreads / 2; stride >= 1; stride >>= 1) {
+    if (threadIdx.x < stride) {
+      sa[threadIdx.x] += sa[threadIdx.x + stride];
+      sb[threadIdx.x] += sb[threadIdx.x + stride];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    out_a[c] = sa[0];
+    out_b[c] = sb[0];
+  }
+}
+
+// qstats[0] = max over all entries of max(|q.grad|, q.hess); qstats[1] != 0 if a
+// value does not fit the packed int32 form.
+__global__ void scales_kernel(const double* sum_a, const double* sum_b, double* scales,
+                              unsigned long long* qstats)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const double max_int = 2147483647.0;
+    double sg = sum_a[0] == 0 ? 1 : max_int / sum_a[0];
+    double sh = sum_b[0] == 0 ? 1 : max_int / sum_b[0];
+    scales[0] = sg;
+    scales[1] = sh;
+    scales[2] = 1.0 / sg;
+    scales[3] = 1.0 / sh;
+    qstats[0] = 0;
+    qstats[1] = 0;
+  }
+}
+
+// Stochastic rounding of every (row, output) once per tree, stored as int32
+// pairs, plus the root sums (build_tree.cu:112-129, :168-204). The reference
+// redoes this rounding inside every histogram launch; the values are the same.
+__global__ void __launch_bounds__(kThreads)
+  quantise_kernel(const double* g, const double* h, int64_t n_rows, int K, int64_t row_offset,
+                  int64_t seed, const double* scales, int2* q_out, I64Pair* node_sums,
+                  unsigned long long* qstats)
+{
+  __shared__ int64_t s_g[kThreads / 64];
+  __shared__ int64_t s_h[kThreads / 64];
+  __shared__ unsigned long long s_m[kThreads / 64];
+  const int k       = blockIdx.y;
+  const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  int64_t qg = 0, qh = 0;
+  unsigned long long mx = 0;
+  bool bad = false;
+  if (row < n_rows) {
+    const double sg = scales[0], sh = scales[1];
+    double grad = g[row * K + k], hess = h[row * K + k];
+    uint32_t x  = minstd_seed(static_cast<uint32_t>(
+      static_cast<uint64_t>(gpair_seed(seed, row + row_offset, static_cast<int64_t>(k)))));
+    double scaled_grad    = grad * sg;
+    double scaled_hess    = hess * sh;
+    double grad_remainder = scaled_grad - floor(scaled_grad);
+    double hess_remainder = scaled_hess - floor(scaled_hess);
+    x  = minstd_next(x);
+    qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
+    x  = minstd_next(x);
+    qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
+    bad = qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
+    q_out[row * K + k] = make_int2(static_cast<int>(qg), static_cast<int>(qh));
+    unsigned long long ag = static_cast<unsigned long long>(qg < 0 ? -qg : qg);
+    unsigned long long ah = static_cast<unsigned long long>(qh < 0 ? -qh : qh);
+    mx = ag > ah ? ag : ah;
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    qg += __shfl_down(qg, off, 64);
+    qh += __shfl_down(qh, off, 64);
+    unsigned long long o = __shfl_down(mx, off, 64);
+    mx = o > mx ? o : mx;
+  }
+  if (bad) atomicMax(&qstats[1], 1ULL);
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (lane == 0) {
+    s_g[wave] = qg;
+    s_h[wave] = qh;
+    s_m[wave] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / 64; w++) {
+      qg += s_g[w];
+      qh += s_h[w];
+      mx = s_m[w] > mx ? s_m[w] : mx;
+    }
+    atomic_add_i64(&node_sums[k].grad, qg);
+    atomic_add_i64(&node_sums[k].hess, qh);
+    atomicMax(&qstats[0], mx);
+  }
+}
+
+// build_tree.cu:1175-1185
+__global__ void root_leaf_kernel(double* leaf, const I64Pair* node_sums, int K,
+                                 const double* scales, double l1, double l2)
+{
+  int k = blockIdx.x * blockDim.x + threadIdx.x;
+  if (k < K) {
+    double G = static_cast<double>(node_sums[k].grad) * scales[2];
+    double H = static_cast<double>(node_sums[k].hess) * scales[3];
+    leaf[k]  = calculate_leaf_value(G, H, l1, l2);
+  }
+}
+
+// build_tree.cu:967-974
+__global__ void fill_positions_kernel(int2* pos, int64_t n)
+{
+  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i < n) pos[i] = make_int2(0, static_cast<int>(i));
+}
+
+// ---------------------------------------------------------------------------
+// histogram
+// ---------------------------------------------------------------------------
+
+constexpr int kHistThreads  = 512;
+constexpr int kTileRows     = 1024;  // rows of one node handled between two bookkeeping steps
+constexpr int kSmallNodeRows = 64;   // below this a node goes straight to global atomics
+constexpr int kHistUnroll   = 4;
+
+struct LevelMeta {
+  int32_t n_tiles;
+  int32_t pad;
+  long long instances;        // rows in the batch
+  long long built_instances;  // rows whose node's histogram is built
+  long long built_nodes;
+};
+
+// For the nodes [j0, j1) of the current level (level-local indices): decides
+// which are built (build_tree.h:92-104) and cuts their row segments into tiles.
+// tile_start[j - j0] = first tile of node j; tile_start[j1 - j0] = total.
+__global__ void __launch_bounds__(kThreads)
+  plan_tiles_kernel(int j0, int j1, int level_first, const int32_t* seg, const I64Pair* node_sums,
+                    int K, int hist_node_begin, int hist_node_end, int32_t* tile_start,
+                    LevelMeta* meta, LevelMeta* level_total)
+{
+  __shared__ int s_scan[kThreads];
+  __shared__ int s_run;
+  __shared__ unsigned long long s_rb, s_rc, s_nb;
+  if (threadIdx.x == 0) {
+    s_run = 0;
+    s_rb = s_rc = s_nb = 0;
+  }
+  __syncthreads();
+  for (int base = j0; base < j1; base += kThreads) {
+    int j      = base + threadIdx.x;
+    int tiles  = 0;
+    int rows   = 0;
+    bool built = false;
+    if (j < j1) {
+      int node   = level_first + j;
+      rows       = seg[j + 1] - seg[j];
+      int parent = parent_of(node);
+      bool pex   = parent >= hist_node_begin && parent < hist_node_end;
+      built      = compute_histogram_bin(node, node_sums, K, pex);
+      tiles      = built ? (rows + kTileRows - 1) / kTileRows : 0;
+    }
+    s_scan[threadIdx.x] = tiles;
+    __syncthreads();
+    // inclusive scan (Hillis-Steele) over the 256 counts
+    for (int off = 1; off < kThreads; off <<= 1) {
+      int v = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
+      __syncthreads();
+      s_scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    int run = s_run;
+    if (j < j1) {
+      tile_start[j - j0] = run + s_scan[threadIdx.x] - tiles;
+      atomicAdd(&s_rb, static_cast<unsigned long long>(rows));
+      if (built && rows > 0) {
+        atomicAdd(&s_rc, static_cast<unsigned long long>(rows));
+        atomicAdd(&s_nb, 1ULL);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == kThreads - 1) s_run = run + s_scan[kThreads - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    tile_start[j1 - j0]   = s_run;
+    meta->n_tiles         = s_run;
+    meta->instances       = s_rb;
+    meta->built_instances = s_rc;
+    meta->built_nodes     = s_nb;
+    level_total->instances += s_rb;
+    level_total->built_instances += s_rc;
+    level_total->built_nodes += s_nb;
+  }
+}
+
+template <typename T>
+struct HistArgs {
+  const T* X;
+  int F;
+  const int2* qgh;  // [N][K] packed int32 (grad, hess)
+  int K;
+  const int2* positions;  // (node,row) sorted by node
+  const int32_t* seg;     // level-local segment starts
+  int j0;                 // first level-local node of the batch
+  int n_nodes;            // nodes in the batch
+  int level_first;        // global index of level-local node 0
+  const int32_t* tile_start;
+  const LevelMeta* meta;
+  const T* proposals;
+  const int32_t* row_pointers;
+  const int32_t* groups;  // feature groups: [n_groups+1]
+  int search_steps;       // ceil(log2(max bins of one feature))
+  HistView hist;
+  const unsigned long long* qstats;
+};
+
+// Number of proposals of [p, p+n) that are < x, i.e. lower_bound
+// (build_tree.h:178-185), as a fixed-trip-count branch-free search.
+template <typename T>
+__device__ inline int count_less(const T* p, int n, T x, int steps)
+{
+  int lo = 0;
+  for (int s = 0; s < steps; s++) {
+    int half = n >> 1;
+    bool go  = n > 0 && p[lo + half] < x;
+    lo       = go ? lo + half + 1 : lo;
+    n        = go ? n - half - 1 : half;
+  }
+  return lo;
+}
+
+// One workgroup owns (a contiguous range of row tiles) x (one feature group) x
+// (one output). Thread t is tied to feature f0 + t % gs for its whole life and
+// walks rows t / gs, t / gs + rows_per_pass, ...: the lanes of a wave read
+// consecutive features of a row (contiguous bytes), and the per-feature search
+// range lives in registers. Sums go to an int32 sub-histogram in LDS and are
+// merged into the int64 histogram with global atomics when the node changes
+// (reference: fill_histogram_shared, build_tree.cu:213-480).
+template <typename T>
+__global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
+{
+  extern __shared__ unsigned char smem_raw[];
+  const int group = blockIdx.y;
+  const int k     = blockIdx.z;
+  const int f0 = a.groups[group], f1 = a.groups[group + 1];
+  const int gs   = f1 - f0;
+  const int bin0 = a.row_pointers[f0];
+  const int nb   = a.row_pointers[f1] - bin0;
+  T* s_prop          = reinterpret_cast<T*>(smem_raw);
+  uint32_t* s_hist   = reinterpret_cast<uint32_t*>(smem_raw + ((static_cast<size_t>(nb) * sizeof(T) + 15) & ~size_t(15)));
+
+  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_prop[i] = a.proposals[bin0 + i];
+  for (int i = threadIdx.x; i < 2 * nb; i += kHistThreads) s_hist[i] = 0;
+
+  const int rows_per_pass = kHistThreads / gs;
+  const bool active       = static_cast<int>(threadIdx.x) < rows_per_pass * gs;
+  const int fl            = threadIdx.x % gs;
+  const int rsub          = threadIdx.x / gs;
+  const int f             = f0 + fl;
+  const int pbase         = a.row_pointers[f] - bin0;
+  const int pn            = a.row_pointers[f + 1] - a.row_pointers[f];
+  const unsigned long long max_abs = a.qstats[0];
+
+  const int n_tiles = a.meta->n_tiles;
+  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * blockIdx.x / gridDim.x);
+  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (blockIdx.x + 1) / gridDim.x);
+
+  int cur_node           = -1;
+  unsigned long long acc = 0;  // rows added to the LDS copy since it was last cleared
+  __syncthreads();
+
+  auto flush = [&](int node) {
+    __syncthreads();
+    if (node >= 0) {
+      I64Pair* dst = a.hist.at(node, k, bin0);
+      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+        int32_t gv  = static_cast<int32_t>(s_hist[2 * i]);
+        uint32_t hv = s_hist[2 * i + 1];
+        if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
+        if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
+        s_hist[2 * i]     = 0;
+        s_hist[2 * i + 1] = 0;
+      }
+    }
+    __syncthreads();
+  };
+
+  for (int tile = t_begin; tile < t_end; tile++) {
+    // node of this tile: last j with tile_start[j] <= tile (uniform over the block)
+    int lo = 0, hi = a.n_nodes;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (a.tile_start[mid] <= tile)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
+    const int j        = a.j0 + lo;
+    const int node     = a.level_first + j;
+    const int seg_lo   = a.seg[j];
+    const int seg_hi   = a.seg[j + 1];
+    const int r0       = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
+    const int r1       = min(seg_hi, r0 + kTileRows);
+    const int nrows    = r1 - r0;
+    const bool direct  = (seg_hi - seg_lo) < kSmallNodeRows ||
+                        static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
+    if (!direct) {
+      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
+        flush(cur_node);
+        cur_node = node;
+        acc      = 0;
+      }
+      acc += nrows;
+    }
+    if (active) {
+      I64Pair* gdst = a.hist.at(node, k, bin0);
+      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kHistUnroll) {
+        int row[kHistUnroll];
+        T x[kHistUnroll];
+        int2 q[kHistUnroll];
+#pragma unroll
+        for (int u = 0; u < kHistUnroll; u++) {
+          int rr = r + u * rows_per_pass;
+          row[u] = rr < r1 ? a.positions[rr].y : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < kHistUnroll; u++) {
+          if (row[u] >= 0) {
+            x[u] = a.X[static_cast<int64_t>(row[u]) * a.F + f];
+            q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kHistUnroll; u++) {
+          if (row[u] >= 0) {
+            int bin = pbase + count_less(s_prop + pbase, pn, x[u], a.search_steps);
+            if (direct) {
+              atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
+              atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
+            } else {
+              atomicAdd(&s_hist[2 * bin], static_cast<uint32_t>(q[u].x));
+              atomicAdd(&s_hist[2 * bin + 1], static_cast<uint32_t>(q[u].y));
+            }
+          }
+        }
+      }
+    }
+  }
+  flush(cur_node);
+}
+
+// ---------------------------------------------------------------------------
+// scan + sibling subtraction (build_tree.cu:597-668), one wave per
+// (feature, node), 64 bins per step
+// ---------------------------------------------------------------------------
+
+__global__ void __launch_bounds__(kThreads)
+  scan_kernel(HistView hist, const I64Pair* node_sums, int F, const int32_t* row_pointers,
+              int node_begin, int n_nodes)
+{
+  const int lane     = threadIdx.x & 63;
+  const int64_t rank = (blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x) >> 6;
+  const int i        = static_cast<int>(rank / n_nodes);
+  const int j        = static_cast<int>(rank % n_nodes);
+  const int k        = blockIdx.y;
+  if (i >= F) return;
+  const int node   = node_begin + j;
+  const int parent = parent_of(node);
+  if (node_sums[static_cast<int64_t>(node) * hist.K + k].hess <= 0) return;
+  if (!compute_histogram_bin(node, node_sums, hist.K, hist.contains(parent))) return;
+
+  const int fb = row_pointers[i], fe = row_pointers[i + 1];
+  int64_t agg_g = 0, agg_h = 0;
+  for (int base = fb; base < fe; base += 64) {
+    const int bin  = base + lane;
+    const bool in  = bin < fe;
+    I64Pair* cell  = hist.at(node, k, in ? bin : fb);
+    int64_t eg = in ? cell->grad : 0, eh = in ? cell->hess : 0;
+    for (int off = 1; off < 64; off <<= 1) {
+      int64_t og = __shfl_up(eg, off, 64);
+      int64_t oh = __shfl_up(eh, off, 64);
+      if (lane >= off) {
+        eg += og;
+        eh += oh;
+      }
+    }
+    int64_t tile_g = __shfl(eg, 63, 64), tile_h = __shfl(eh, 63, 64);
+    eg += agg_g;
+    eh += agg_h;
+    // the reference skips the store when the running sum is not positive
+    // (build_tree.cu:645); the raw bin value then stays in place
+    if (in && (eg > 0 || eh > 0)) {
+      cell->grad = eg;
+      cell->hess = eh;
+    }
+    agg_g += tile_g;
+    agg_h += tile_h;
+  }
+  if (node == 0) return;
+  const int sib = sibling_of(node);
+  if (!compute_histogram_bin(sib, node_sums, hist.K, hist.contains(parent))) {
+    for (int bin = fb + lane; bin < fe; bin += 64) {
+      I64Pair s = *hist.at(node, k, bin);
+      I64Pair p = *hist.at(parent, k, bin);
+      *hist.at(sib, k, bin) = I64Pair{p.grad - s.grad, p.hess - s.hess};
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// split evaluation (build_tree.cu:682-782)
+// ---------------------------------------------------------------------------
+
+struct Cand {
+  double gain;
+  int bin;
+};
+
+// Total order equivalent to the reference's 512 strided threads followed by a
+// rank-ordered reduction with op(a,b) = a.gain > b.gain ? a : b: larger gain
+// wins; among equal gains the larger (bin mod 512); inside one residue class
+// the smaller bin. Only bins with gain > 0 are candidates.
+__device__ inline bool cand_better(const Cand& a, const Cand& b)
+{
+  if (a.bin < 0) return false;
+  if (b.bin < 0) return true;
+  if (a.gain != b.gain) return a.gain > b.gain;
+  int ra = a.bin & 511, rb = b.bin & 511;
+  if (ra != rb) return ra > rb;
+  return a.bin < b.bin;
+}
+
+constexpr int kSplitChunk = 2048;  // bins per workgroup
+
+__device__ inline Cand block_best(Cand c, Cand* s_c)
+{
+  for (int off = 32; off >= 1; off >>= 1) {
+    Cand o;
+    o.gain = __shfl_down(c.gain, off, 64);
+    o.bin  = __shfl_down(c.bin, off, 64);
+    if (cand_better(o, c)) c = o;
+  }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) s_c[wave] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < static_cast<int>(blockDim.x) >> 6; w++)
+      if (cand_better(s_c[w], c)) c = s_c[w];
+  }
+  return c;  // valid on thread 0
+}
+
+__global__ void __launch_bounds__(kThreads)
+  split_eval_kernel(HistView hist, const I64Pair* node_sums, const int32_t* bin_feature,
+                    const uint8_t* feature_set, const double* scales, double l1, double l2,
+                    double min_split_gain, int node_begin, int n_chunks, Cand* partial)
+{
+  __shared__ Cand s_c[kThreads / 64];
+  const int node = node_begin + blockIdx.x;
+  const int K    = hist.K;
+  if (node_sums[static_cast<int64_t>(node) * K].hess <= 0) return;
+  const double inv_g = scales[2], inv_h = scales[3];
+  const double reg   = 1e-5 > l2 ? 1e-5 : l2;
+  const int b_lo     = blockIdx.y * kSplitChunk;
+  const int b_hi     = min(hist.B, b_lo + kSplitChunk);
+  Cand best{0.0, -1};
+  for (int bin = b_lo + threadIdx.x; bin < b_hi; bin += kThreads) {
+    if (feature_set != nullptr && !feature_set[bin_feature[bin]]) continue;
+    double gain = 0;
+    for (int k = 0; k < K; k++) {
+      I64Pair ns = node_sums[static_cast<int64_t>(node) * K + k];
+      I64Pair ls = *hist.at(node, k, bin);
+      int64_t rg = ns.grad - ls.grad, rh = ns.hess - ls.hess;
+      if (ls.hess <= 0 || rh <= 0) {
+        gain = 0;
+        break;
+      }
+      gain += calculate_gain(static_cast<double>(ls.grad) * inv_g, static_cast<double>(ls.hess) * inv_h,
+                             static_cast<double>(rg) * inv_g, static_cast<double>(rh) * inv_h,
+                             static_cast<double>(ns.grad) * inv_g, static_cast<double>(ns.hess) * inv_h,
+                             l1, reg, min_split_gain);
+    }
+    if (gain > 0) {
+      Cand c{gain, bin};
+      if (cand_better(c, best)) best = c;
+    }
+  }
+  best = block_best(best, s_c);
+  if (threadIdx.x == 0) partial[static_cast<int64_t>(blockIdx.x) * n_chunks + blockIdx.y] = best;
+}
+
+__global__ void __launch_bounds__(64)
+  split_apply_kernel(HistView hist, I64Pair* node_sums, const int32_t* bin_feature,
+                     const double* proposals_as_double, const double* scales, double l1, double l2,
+                     int node_begin, int n_chunks, const Cand* partial, double* leaf,
+                     int32_t* feature, double* split, double* gain_out)
+{
+  __shared__ Cand s_c[1];
+  __shared__ Cand s_best;
+  const int node = node_begin + blockIdx.x;
+  const int K    = hist.K;
+  if (node_sums[static_cast<int64_t>(node) * K].hess <= 0) return;
+  Cand best{0.0, -1};
+  for (int c = threadIdx.x; c < n_chunks; c += 64) {
+    Cand o = partial[static_cast<int64_t>(blockIdx.x) * n_chunks + c];
+    if (cand_better(o, best)) best = o;
+  }
+  best = block_best(best, s_c);
+  if (threadIdx.x == 0) s_best = best;
+  __syncthreads();
+  best = s_best;
+  if (!(best.bin >= 0 && best.gain > 1e-5)) return;
+  const double inv_g = scales[2], inv_h = scales[3];
+  const int lc = left_child(node), rc = right_child(node);
+  for (int k = threadIdx.x; k < K; k += 64) {
+    I64Pair ns = node_sums[static_cast<int64_t>(node) * K + k];
+    I64Pair ls = *hist.at(node, k, best.bin);
+    I64Pair rs{ns.grad - ls.grad, ns.hess - ls.hess};
+    node_sums[static_cast<int64_t>(lc) * K + k] = ls;
+    node_sums[static_cast<int64_t>(rc) * K + k] = rs;
+    leaf[static_cast<int64_t>(lc) * K + k] = calculate_leaf_value(
+      static_cast<double>(ls.grad) * inv_g, static_cast<double>(ls.hess) * inv_h, l1, l2);
+    leaf[static_cast<int64_t>(rc) * K + k] = calculate_leaf_value(
+      static_cast<double>(rs.grad) * inv_g, static_cast<double>(rs.hess) * inv_h, l1, l2);
+    if (k == 0) {
+      feature[node]  = bin_feature[best.bin];
+      split[node]    = proposals_as_double[best.bin];
+      gain_out[node] = best.gain;
+    }
+  }
+}
+
+template <typename T>
+__global__ void proposals_to_double_kernel(const T* p, int n, double* out)
+{
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = static_cast<double>(p[i]);
+}
+
+// ---------------------------------------------------------------------------
+// row -> node update and stable partition (build_tree.cu:1026-1080)
+// ---------------------------------------------------------------------------
+//
+// The reference rewrites the node of every (node,row) pair and then runs a
+// stable radix sort on the node field. Because the pairs are already sorted by
+// node and a node only splits into its two children (or its rows retire with
+// key -1), that sort is a stable three-way partition inside every segment:
+// retired rows move to the front, then for each parent its left rows followed
+// by its right rows. Exclusive prefix counts of the "retired" and "left" flags
+// give every destination directly.
+
+constexpr int kPartItems = 4;
+constexpr int kPartBlock = kThreads * kPartItems;  // rows per workgroup
+
+// pass 1: classify each row (0 retired, 1 left, 2 right) and count per workgroup
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+  classify_kernel(const int2* pos, int64_t n, const T* X, int F, const int32_t* feature,
+                  const double* split, int max_nodes, uint8_t* code, int2* block_counts)
+{
+  __shared__ int s_d[kThreads / 64];
+  __shared__ int s_l[kThreads / 64];
+  const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  int nd = 0, nl = 0;
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    int64_t i = base + u * kThreads + threadIdx.x;
+    if (i < n) {
+      int2 p = pos[i];
+      int c  = 0;
+      if (p.x >= 0 && p.x < max_nodes) {
+        int ft = feature[p.x];
+        if (ft != -1) {
+          double xv = static_cast<double>(X[static_cast<int64_t>(p.y) * F + ft]);
+          c         = xv <= split[p.x] ? 1 : 2;
+        }
+      }
+      code[i] = static_cast<uint8_t>(c);
+      nd += c == 0;
+      nl += c == 1;
+    }
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    nd += __shfl_down(nd, off, 64);
+    nl += __shfl_down(nl, off, 64);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_d[threadIdx.x >> 6] = nd;
+    s_l[threadIdx.x >> 6] = nl;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / 64; w++) {
+      nd += s_d[w];
+      nl += s_l[w];
+    }
+    block_counts[blockIdx.x] = make_int2(nd, nl);
+  }
+}
+
+// pass 2: exclusive scan of the per-workgroup counts (single workgroup)
+__global__ void __launch_bounds__(kThreads)
+  scan_block_counts_kernel(const int2* block_counts, int n_blocks, int2* block_offsets, int2* totals)
+{
+  __shared__ int s_d[kThreads];
+  __shared__ int s_l[kThreads];
+  __shared__ int run_d, run_l;
+  if (threadIdx.x == 0) run_d = run_l = 0;
+  __syncthreads();
+  for (int base = 0; base < n_blocks; base += kThreads) {
+    int b   = base + threadIdx.x;
+    int2 c  = b < n_blocks ? block_counts[b] : make_int2(0, 0);
+    s_d[threadIdx.x] = c.x;
+    s_l[threadIdx.x] = c.y;
+    __syncthreads();
+    for (int off = 1; off < kThreads; off <<= 1) {
+      int vd = threadIdx.x >= off ? s_d[threadIdx.x - off] : 0;
+      int vl = threadIdx.x >= off ? s_l[threadIdx.x - off] : 0;
+      __syncthreads();
+      s_d[threadIdx.x] += vd;
+      s_l[threadIdx.x] += vl;
+      __syncthreads();
+    }
+    if (b < n_blocks) block_offsets[b] = make_int2(run_d + s_d[threadIdx.x] - c.x, run_l + s_l[threadIdx.x] - c.y);
+    __syncthreads();
+    if (threadIdx.x == kThreads - 1) {
+      run_d += s_d[kThreads - 1];
+      run_l += s_l[kThreads - 1];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *totals = make_int2(run_d, run_l);
+}
+
+// Prefix counts (retired, left) in front of index s.
+__device__ inline int2 prefix_at(int s, int64_t n, const uint8_t* code, const int2* block_offsets,
+                                 const int2* totals, int lane)
+{
+  if (s >= n) return *totals;
+  int b      = s / kPartBlock;
+  int2 off   = block_offsets[b];
+  int nd = 0, nl = 0;
+  for (int i = b * kPartBlock + lane; i < s; i += 64) {
+    int c = code[i];
+    nd += c == 0;
+    nl += c == 1;
+  }
+  for (int o = 32; o >= 1; o >>= 1) {
+    nd += __shfl_xor(nd, o, 64);
+    nl += __shfl_xor(nl, o, 64);
+  }
+  return make_int2(off.x + nd, off.y + nl);
+}
+
+// pass 3: one wave per parent j: prefix counts at its segment start, and the
+// segment starts of its two children in the next level.
+__global__ void __launch_bounds__(kThreads)
+  child_segments_kernel(const int32_t* seg, int n_parents, int64_t n, const uint8_t* code,
+                        const int2* block_offsets, const int2* totals, int2* seg_prefix,
+                        int32_t* seg_next)
+{
+  const int lane = threadIdx.x & 63;
+  const int j    = static_cast<int>((blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x) >> 6);
+  if (j >= n_parents) return;
+  int s0 = seg[j], s1 = seg[j + 1];
+  int2 p0 = prefix_at(s0, n, code, block_offsets, totals, lane);
+  int2 p1 = prefix_at(s1, n, code, block_offsets, totals, lane);
+  if (lane == 0) {
+    int total_dead      = totals->x;
+    int base            = total_dead + (s0 - p0.x);
+    seg_prefix[j]       = p0;
+    seg_next[2 * j]     = base;
+    seg_next[2 * j + 1] = base + (p1.y - p0.y);
+    if (j == n_parents - 1) seg_next[2 * n_parents] = static_cast<int32_t>(n);
+  }
+}
+
+// pass 4: scatter every pair to its place in the next level's order
+__global__ void __launch_bounds__(kThreads)
+  scatter_kernel(const int2* pos, int64_t n, const uint8_t* code, const int2* block_offsets,
+                 const int32_t* seg, const int2* seg_prefix, const int32_t* seg_next,
+                 int level_first, int n_parents, int2* pos_out)
+{
+  __shared__ int s_wave[kThreads / 64];
+  const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // thread t owns the kPartItems consecutive rows base + t*kPartItems ...
+  int2 p[kPartItems];
+  int c[kPartItems];
+  int packed = 0;  // retired count in the high half, left count in the low half
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    int64_t i = base + static_cast<int64_t>(threadIdx.x) * kPartItems + u;
+    c[u]      = 3;
+    if (i < n) {
+      p[u] = pos[i];
+      c[u] = code[i];
+      packed += (c[u] == 0 ? (1 << 16) : 0) + (c[u] == 1 ? 1 : 0);
+    }
+  }
+  int incl = packed;
+  for (int off = 1; off < 64; off <<= 1) {
+    int o = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int w = 0; w < kThreads / 64; w++) {
+      int v     = s_wave[w];
+      s_wave[w] = run;
+      run += v;
+    }
+  }
+  __syncthreads();
+  int excl   = s_wave[wave] + incl - packed;
+  int2 boff  = block_offsets[blockIdx.x];
+  int D      = boff.x + (excl >> 16);
+  int L      = boff.y + (excl & 0xffff);
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    int64_t i = base + static_cast<int64_t>(threadIdx.x) * kPartItems + u;
+    if (i < n) {
+      int dest;
+      int new_node;
+      if (c[u] == 0) {
+        dest     = D;
+        new_node = -1;
+        D++;
+      } else {
+        int j       = p[u].x - level_first;
+        int s0      = seg[j];
+        int2 sp     = seg_prefix[j];
+        if (c[u] == 1) {
+          dest     = seg_next[2 * j] + (L - sp.y);
+          new_node = left_child(p[u].x);
+          L++;
+        } else {
+          int R    = static_cast<int>(i) - D - L;
+          int R0   = s0 - sp.x - sp.y;
+          dest     = seg_next[2 * j + 1] + (R - R0);
+          new_node = right_child(p[u].x);
+        }
+      }
+      pos_out[dest] = make_int2(new_node, p[u].y);
+    }
+  }
+}
+
+__global__ void init_seg_kernel(int32_t* seg, int32_t n)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    seg[0] = 0;
+    seg[1] = n;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+
+struct Layout {
+  // tree state
+  I64Pair* node_sums;
+  double* scales;
+  unsigned long long* qstats;
+  // proposals
+  void* draft;
+  void* uniq;
+  int32_t* counts;
+  void* proposals;
+  double* proposals_d;
+  int32_t* row_pointers;
+  int32_t* bin_feature;
+  int32_t* groups;
+  // quantiser
+  double* part_a[2];
+  double* part_b[2];
+  int2* qgh;
+  // positions
+  int2* pos[2];
+  int32_t* seg[2];
+  uint8_t* code;
+  int2* block_counts;
+  int2* block_offsets;
+  int2* totals;
+  int2* seg_prefix;
+  // histogram
+  int32_t* tile_start;
+  LevelMeta* meta;
+  LevelMeta* level_totals;
+  Cand* partial;
+  I64Pair* hist;
+  size_t hist_bytes;
+};
+
+size_t hist_bytes_bound(int F, int K, int S, int max_depth, int64_t cache_bytes)
+{
+  if (max_depth < 1) return 0;
+  const double bpn = static_cast<double>(K) * F * S * 16.0;  // bytes per node with every bin distinct
+  const double max_bytes = cache_bytes > 0 ? static_cast<double>(cache_bytes) : 1e9;
+  double a = std::max(max_bytes, bpn);
+  double b = static_cast<double>(level_end(max_depth - 1)) * bpn;
+  return static_cast<size_t>(std::min(a, b)) + 256;
+}
+
+void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, int S,
+                 size_t elem, int64_t cache_bytes)
+{
+  const int64_t max_nodes   = level_end(max_depth);
+  const int64_t level_nodes = int64_t(1) << (max_depth > 0 ? max_depth - 1 : 0);
+  L.node_sums    = ar.take<I64Pair>(max_nodes * K);
+  L.scales       = ar.take<double>(4);
+  L.qstats       = ar.take<unsigned long long>(2);
+  L.draft        = ar.take<char>(static_cast<size_t>(F) * S * elem);
+  L.uniq         = ar.take<char>(static_cast<size_t>(F) * S * elem);
+  L.counts       = ar.take<int32_t>(F);
+  L.proposals    = ar.take<char>(static_cast<size_t>(F) * S * elem);
+  L.proposals_d  = ar.take<double>(static_cast<size_t>(F) * S);
+  L.row_pointers = ar.take<int32_t>(F + 1);
+  L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
+  L.groups       = ar.take<int32_t>(F + 1);
+  int64_t n_chunks = (N * K + 4095) / 4096;
+  for (int i = 0; i < 2; i++) {
+    L.part_a[i] = ar.take<double>(n_chunks);
+    L.part_b[i] = ar.take<double>(n_chunks);
+    n_chunks    = (n_chunks + 4095) / 4096;
+  }
+  L.qgh    = ar.take<int2>(N * K);
+  L.pos[0] = ar.take<int2>(N);
+  L.pos[1] = ar.take<int2>(N);
+  L.seg[0] = ar.take<int32_t>(level_nodes + 1);
+  L.seg[1] = ar.take<int32_t>(level_nodes + 1);
+  L.code   = ar.take<uint8_t>(N);
+  const int64_t n_pblocks = (N + kPartBlock - 1) / kPartBlock;
+  L.block_counts  = ar.take<int2>(n_pblocks);
+  L.block_offsets = ar.take<int2>(n_pblocks);
+  L.totals        = ar.take<int2>(1);
+  L.seg_prefix    = ar.take<int2>(level_nodes);
+  L.tile_start    = ar.take<int32_t>(level_nodes + 1);
+  L.meta          = ar.take<LevelMeta>(1);
+  L.level_totals  = ar.take<LevelMeta>(max_depth > 0 ? max_depth : 1);
+  const int64_t max_chunks = (static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk;
+  L.partial       = ar.take<Cand>(level_nodes * max_chunks);
+  L.hist_bytes    = hist_bytes_bound(F, K, S, max_depth, cache_bytes);
+  L.hist          = reinterpret_cast<I64Pair*>(ar.take<char>(L.hist_bytes));
+}
+
+int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
+{
+  LBT_REQUIRE(p != nullptr, "params is null");
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(N >= 1 && N < 2147483647LL, "n_rows %lld out of range", static_cast<long long>(N));
+  LBT_REQUIRE(F >= 1 && K >= 1, "n_features and n_outputs must be positive");
+  LBT_REQUIRE(K <= 65535, "n_outputs above 65535 is not supported");
+  LBT_REQUIRE(p->max_depth >= 0 && p->max_depth <= 24, "max_depth %d out of range [0,24]", p->max_depth);
+  LBT_REQUIRE(static_cast<int64_t>(p->max_nodes) == level_end(p->max_depth),
+              "max_nodes must be 2^(max_depth+1)-1");
+  LBT_REQUIRE(p->split_samples >= 1 && p->split_samples <= LBT_MAX_SPLIT_SAMPLES,
+              "split_samples must be in [1, %d]", LBT_MAX_SPLIT_SAMPLES);
+  LBT_REQUIRE(p->dataset_rows >= 1, "dataset_rows must be positive");
+  LBT_REQUIRE(p->hist_cache_bytes >= 0, "hist_cache_bytes must not be negative");
+  return LBT_OK;
+}
+
+constexpr size_t kHistLdsBudget = 64 * 1024;
+
+template <typename T>
+int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F,
+                    const double* g, const double* h, int K, const uint8_t* feature_set,
+                    const lbt_build_params& prm, double* leaf, int32_t* feature, double* split,
+                    double* gain, double* hessian, Layout& L, lbt_build_taps* taps)
+{
+  const int max_depth = prm.max_depth;
+  const int max_nodes = prm.max_nodes;
+  const int S         = prm.split_samples;
+  auto blocks = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+
+  {
+    ProfScope ps(LBT_PROF_OTHER, stream);
+    init_tree_kernel<<<blocks(static_cast<int64_t>(max_nodes) * K, kThreads), kThreads, 0, stream>>>(
+      leaf, feature, split, gain, L.node_sums, max_nodes, K);
+  }
+
+  // ---- split proposals
+  std::vector<int32_t> rp(F + 1);
+  {
+    ProfScope ps(LBT_PROF_PROPOSALS, stream);
+    T* draft = static_cast<T*>(L.draft);
+    T* uniq  = static_cast<T*>(L.uniq);
+    gather_samples_kernel<T><<<blocks(static_cast<int64_t>(F) * S, kThreads), kThreads, 0, stream>>>(
+      X, row_offset, N, F, S, prm.seed, prm.dataset_rows, draft);
+    int P = 1;
+    while (P < S) P <<= 1;
+    if (P < 2) P = 2;
+    sort_unique_kernel<T><<<F, kThreads, P * sizeof(typename KeyOf<T>::type), stream>>>(
+      draft, S, P, uniq, L.counts);
+    row_pointers_kernel<<<1, 64, 0, stream>>>(L.counts, F, L.row_pointers);
+    compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(
+      uniq, S, L.row_pointers, static_cast<T*>(L.proposals), L.bin_feature);
+    LBT_HIP(hipMemcpyAsync(rp.data(), L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
+  }
+  LBT_HIP(hipStreamSynchronize(stream));
+  const int B = rp[F];
+  proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
+    static_cast<const T*>(L.proposals), B, L.proposals_d);
+
+  // feature groups: consecutive features packed while proposals + int32
+  // sub-histogram fit the LDS budget and the group is not wider than a workgroup
+  std::vector<int32_t> groups{0};
+  int max_feature_bins = 1;
+  size_t lds_bytes     = 0;
+  {
+    const size_t per_bin = sizeof(T) + 8;
+    const int max_bins   = static_cast<int>((kHistLdsBudget - 16) / per_bin);
+    // balance: aim at equal-width groups
+    int64_t n_groups_min = (static_cast<int64_t>(B) + max_bins - 1) / max_bins;
+    int target_bins = static_cast<int>((B + n_groups_min - 1) / n_groups_min);
+    int cur = 0, width = 0;
+    for (int f = 0; f < F; f++) {
+      int nb = rp[f + 1] - rp[f];
+      max_feature_bins = std::max(max_feature_bins, nb);
+      if (width > 0 && (cur + nb > max_bins || width >= kHistThreads / 2 ||
+                        (cur >= target_bins))) {
+        groups.push_back(f);
+        cur   = 0;
+        width = 0;
+      }
+      cur += nb;
+      width++;
+    }
+    groups.push_back(F);
+    int gmax = 0;
+    for (size_t i = 0; i + 1 < groups.size(); i++) gmax = std::max(gmax, rp[groups[i + 1]] - rp[groups[i]]);
+    lds_bytes = ((static_cast<size_t>(gmax) * sizeof(T) + 15) & ~size_t(15)) + static_cast<size_t>(gmax) * 8;
+  }
+  const int n_groups = static_cast<int>(groups.size()) - 1;
+  LBT_HIP(hipMemcpyAsync(L.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
+  int search_steps = 0;
+  while ((1 << search_steps) < max_feature_bins + 1) search_steps++;
+
+  // ---- quantiser
+  {
+    ProfScope ps(LBT_PROF_QUANTISE, stream, static_cast<double>(N) * K * (16 + 16 + 8));
+    int64_t n = N * K;
+    int64_t m = (n + 4095) / 4096;
+    abs_sum_level_kernel<true><<<static_cast<unsigned>(m), kThreads, 0, stream>>>(g, h, n, L.part_a[0], L.part_b[0]);
+    int cur = 0;
+    while (m > 1) {
+      int64_t m2 = (m + 4095) / 4096;
+      abs_sum_level_kernel<false><<<static_cast<unsigned>(m2), kThreads, 0, stream>>>(
+        L.part_a[cur], L.part_b[cur], m, L.part_a[cur ^ 1], L.part_b[cur ^ 1]);
+      cur ^= 1;
+      m = m2;
+    }
+    scales_kernel<<<1, 64, 0, stream>>>(L.part_a[cur], L.part_b[cur], L.scales, L.qstats);
+    dim3 grid(blocks(N, kThreads), K);
+    quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(prm.seed),
+                                                   L.scales, L.qgh, L.node_sums, L.qstats);
+    root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
+                                                       prm.l1_regularization, prm.l2_regularization);
+  }
+  unsigned long long h_qstats[2] = {0, 0};
+  LBT_HIP(hipMemcpyAsync(h_qstats, L.qstats, sizeof(h_qstats), hipMemcpyDeviceToHost, stream));
+
+  // ---- positions and histogram cache (TreeBuilder ctor, build_tree.cu:997-1017)
+  fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.pos[0], N);
+  init_seg_kernel<<<1, 64, 0, stream>>>(L.seg[0], static_cast<int32_t>(N));
+  const uint64_t max_bytes = prm.hist_cache_bytes > 0 ? static_cast<uint64_t>(prm.hist_cache_bytes) : 1000000000ULL;
+  const uint64_t bytes_per_node = static_cast<uint64_t>(K) * B * 16ULL;
+  uint64_t max_histogram_nodes  = std::max<uint64_t>(1, max_bytes / bytes_per_node);
+  int cdepth = 0;
+  while (static_cast<uint64_t>(level_end(cdepth + 1)) <= max_histogram_nodes && cdepth <= max_depth) cdepth++;
+  const int64_t max_batch_size = static_cast<int64_t>(static_cast<int>(max_histogram_nodes));
+  // only nodes of levels < max_depth ever get a histogram
+  const int64_t used_end = max_depth > 0 ? level_end(max_depth - 1) : 0;
+  HistView hv{L.hist, 0, static_cast<int>(level_end(cdepth)), K, B};
+  auto zero_hist = [&](int node_begin, int node_end) -> int {
+    int64_t hi    = std::min<int64_t>(node_end, used_end);
+    int64_t nodes = hi - node_begin;
+    if (nodes <= 0) return LBT_OK;
+    uint64_t bytes = static_cast<uint64_t>(nodes) * bytes_per_node;
+    if (bytes > L.hist_bytes) {
+      set_error("histogram workspace too small (%llu > %llu)", (unsigned long long)bytes,
+                (unsigned long long)L.hist_bytes);
+      return LBT_ERR_WORKSPACE;
+    }
+    ProfScope ps(LBT_PROF_OTHER, stream, static_cast<double>(bytes));
+    int64_t n16 = static_cast<int64_t>(bytes / 16);
+    zero_kernel<<<static_cast<unsigned>(std::min<int64_t>((n16 + kThreads - 1) / kThreads, 65536)), kThreads, 0, stream>>>(
+      reinterpret_cast<uint4*>(L.hist), n16);
+    return LBT_OK;
+  };
+  LBT_TRY(zero_hist(hv.node_begin, hv.node_end));
+  static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
+  if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
+
+  LBT_HIP(hipStreamSynchronize(stream));
+  if (h_qstats[1] != 0) {
+    set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
+    return LBT_ERR_UNSUPPORTED;
+  }
+
+  int device = 0, n_cu = 256;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  if (lds_bytes > 48 * 1024)
+    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(histogram_kernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+
+  int cur_pos = 0, cur_seg = 0;
+  const int n_chunks = (B + kSplitChunk - 1) / kSplitChunk;
+  for (int depth = 0; depth < max_depth; depth++) {
+    if (taps && taps->positions_per_level)
+      LBT_HIP(hipMemcpyAsync(taps->positions_per_level + static_cast<size_t>(depth) * N * 2, L.pos[cur_pos],
+                             sizeof(int2) * N, hipMemcpyDeviceToDevice, stream));
+    const int64_t nodes_in_level = int64_t(1) << depth;
+    const int level_first        = static_cast<int>(level_begin(depth));
+    int64_t num_batches          = 1;
+    if (nodes_in_level > max_batch_size) num_batches = (nodes_in_level + max_batch_size - 1) / max_batch_size;
+    for (int64_t bi = 0; bi < num_batches; bi++) {
+      int j0 = 0, j1 = static_cast<int>(nodes_in_level);
+      if (num_batches > 1) {
+        j0 = static_cast<int>(bi * max_batch_size);
+        j1 = static_cast<int>(std::min<int64_t>(j0 + max_batch_size, nodes_in_level));
+      }
+      const int batch_begin = level_first + j0, batch_end = level_first + j1;
+      // GetHistogram (build_tree.cu:1191-1205)
+      if (!(batch_begin >= hv.node_begin && batch_end <= hv.node_end)) {
+        hv.node_begin = batch_begin;
+        hv.node_end   = batch_end;
+        LBT_TRY(zero_hist(hv.node_begin, hv.node_end));
+      }
+      const int n_nodes = j1 - j0;
+      {
+        ProfScope ps(LBT_PROF_OTHER, stream);
+        plan_tiles_kernel<<<1, kThreads, 0, stream>>>(j0, j1, level_first, L.seg[cur_seg], L.node_sums, K,
+                                                      hv.node_begin, hv.node_end, L.tile_start, L.meta,
+                                                      L.level_totals + depth);
+      }
+      {
+        ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
+        HistArgs<T> a;
+        a.X = X; a.F = F; a.qgh = L.qgh; a.K = K; a.positions = L.pos[cur_pos]; a.seg = L.seg[cur_seg];
+        a.j0 = j0; a.n_nodes = n_nodes; a.level_first = level_first; a.tile_start = L.tile_start;
+        a.meta = L.meta; a.proposals = static_cast<const T*>(L.proposals); a.row_pointers = L.row_pointers;
+        a.groups = L.groups; a.search_steps = search_steps; a.hist = hv; a.qstats = L.qstats;
+        // enough workgroups to fill the device, not more than there can be tiles
+        int64_t max_tiles = (N + kTileRows - 1) / kTileRows + n_nodes;
+        int64_t want      = std::max<int64_t>(1, (static_cast<int64_t>(n_cu) * 4) / (static_cast<int64_t>(n_groups) * K));
+        unsigned gx       = static_cast<unsigned>(std::max<int64_t>(1, std::min(max_tiles, want)));
+        dim3 grid(gx, n_groups, K);
+        histogram_kernel<T><<<grid, kHistThreads, lds_bytes, stream>>>(a);
+      }
+      {
+        ProfScope ps(LBT_PROF_SCAN, stream);
+        int64_t waves = static_cast<int64_t>(F) * n_nodes;
+        dim3 grid(blocks(waves, kThreads / 64), K);
+        scan_kernel<<<grid, kThreads, 0, stream>>>(hv, L.node_sums, F, L.row_pointers, batch_begin, n_nodes);
+      }
+      {
+        ProfScope ps(LBT_PROF_SPLIT, stream);
+        dim3 grid(n_nodes, n_chunks);
+        split_eval_kernel<<<grid, kThreads, 0, stream>>>(hv, L.node_sums, L.bin_feature, feature_set, L.scales,
+                                                         prm.l1_regularization, prm.l2_regularization,
+                                                         prm.min_split_gain, batch_begin, n_chunks, L.partial);
+        split_apply_kernel<<<n_nodes, 64, 0, stream>>>(hv, L.node_sums, L.bin_feature, L.proposals_d, L.scales,
+                                                       prm.l1_regularization, prm.l2_regularization, batch_begin,
+                                                       n_chunks, L.partial, leaf, feature, split, gain);
+      }
+    }
+    if (depth < max_depth - 1) {
+      ProfScope ps(LBT_PROF_POSITIONS, stream, static_cast<double>(N) * (8 + 8 + 2 + 64));
+      const unsigned nb = blocks(N, kPartBlock);
+      classify_kernel<T><<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, X, F, feature, split, max_nodes, L.code,
+                                                      L.block_counts);
+      scan_block_counts_kernel<<<1, kThreads, 0, stream>>>(L.block_counts, nb, L.block_offsets, L.totals);
+      const int n_parents = static_cast<int>(nodes_in_level);
+      child_segments_kernel<<<blocks(static_cast<int64_t>(n_parents) * 64, kThreads), kThreads, 0, stream>>>(
+        L.seg[cur_seg], n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[cur_seg ^ 1]);
+      scatter_kernel<<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, L.code, L.block_offsets, L.seg[cur_seg],
+                                                  L.seg_prefix, L.seg[cur_seg ^ 1], level_first, n_parents,
+                                                  L.pos[cur_pos ^ 1]);
+      cur_pos ^= 1;
+      cur_seg ^= 1;
+    }
+  }
+
+  {
+    ProfScope ps(LBT_PROF_OTHER, stream);
+    write_hessian_kernel<<<blocks(static_cast<int64_t>(max_nodes) * K, kThreads), kThreads, 0, stream>>>(
+      hessian, L.node_sums, static_cast<int64_t>(max_nodes) * K, L.scales);
+  }
+
+  // ---- observation points
+  std::vector<LevelMeta> h_levels(max_depth > 0 ? max_depth : 1);
+  const bool want_levels = max_depth > 0 && (profiler().enabled || (taps && (taps->level_instances || taps->level_built_instances || taps->level_built_nodes)));
+  if (want_levels)
+    LBT_HIP(hipMemcpyAsync(h_levels.data(), L.level_totals, sizeof(LevelMeta) * max_depth, hipMemcpyDeviceToHost, stream));
+  if (taps) {
+    taps->n_bins          = B;
+    taps->hist_node_begin = hv.node_begin;
+    taps->hist_node_end   = static_cast<int32_t>(std::max<int64_t>(hv.node_begin, std::min<int64_t>(hv.node_end, used_end)));
+    LBT_HIP(hipMemcpyAsync(taps->scales, L.scales, sizeof(double) * 4, hipMemcpyDeviceToHost, stream));
+    if (taps->proposals)
+      LBT_HIP(hipMemcpyAsync(taps->proposals, L.proposals, sizeof(T) * B, hipMemcpyDeviceToDevice, stream));
+    if (taps->row_pointers)
+      LBT_HIP(hipMemcpyAsync(taps->row_pointers, L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToDevice, stream));
+    if (taps->quantised)
+      LBT_HIP(hipMemcpyAsync(taps->quantised, L.qgh, sizeof(int2) * N * K, hipMemcpyDeviceToDevice, stream));
+    if (taps->node_sums)
+      LBT_HIP(hipMemcpyAsync(taps->node_sums, L.node_sums, sizeof(I64Pair) * max_nodes * K, hipMemcpyDeviceToDevice, stream));
+    if (taps->positions)
+      LBT_HIP(hipMemcpyAsync(taps->positions, L.pos[cur_pos], sizeof(int2) * N, hipMemcpyDeviceToDevice, stream));
+    if (taps->histogram) {
+      int64_t nodes = taps->hist_node_end - taps->hist_node_begin;
+      int64_t need  = nodes * K * B * 2;
+      if (need > 0 && need <= taps->histogram_capacity)
+        LBT_HIP(hipMemcpyAsync(taps->histogram, L.hist, sizeof(int64_t) * need, hipMemcpyDeviceToDevice, stream));
+    }
+  }
+  LBT_HIP(hipStreamSynchronize(stream));
+  LBT_HIP(hipGetLastError());
+  if (want_levels) {
+    for (int d = 0; d < max_depth; d++) {
+      if (taps && taps->level_instances) taps->level_instances[d] = h_levels[d].instances;
+      if (taps && taps->level_built_instances) taps->level_built_instances[d] = h_levels[d].built_instances;
+      if (taps && taps->level_built_nodes) taps->level_built_nodes[d] = static_cast<int32_t>(h_levels[d].built_nodes);
+    }
+  }
+  if (profiler().enabled) {
+    profiler().collect();
+    // algorithmic bytes of the histogram launches of each level:
+    // X rows of built nodes + their packed gradients + one position pair per
+    // instance + the built histograms written once
+    auto& acc = profiler().acc;
+    for (int d = 0; d < max_depth && d < 64; d++) {
+      double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * sizeof(T) + K * 8.0) +
+                  static_cast<double>(h_levels[d].instances) * 8.0 +
+                  static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
+      acc.level_bytes[d] += by;
+      acc.bytes[LBT_PROF_HISTOGRAM] += by;
+    }
+  }
+  return LBT_OK;
+}
+
+}  // namespace
+}  // namespace lbt
+
+extern "C" {
+
+size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_t n_outputs,
+                                      int32_t max_depth, int32_t split_samples, int32_t x_dtype,
+                                      int64_t hist_cache_bytes)
+{
+  lbt_build_params p{};
+  p.max_depth        = max_depth;
+  p.max_nodes        = max_depth >= 0 && max_depth <= 24 ? static_cast<int32_t>(lbt::level_end(max_depth)) : 0;
+  p.split_samples    = split_samples;
+  p.dataset_rows     = 1;
+  p.hist_cache_bytes = hist_cache_bytes;
+  if (lbt::validate(n_rows, n_features, n_outputs, &p, x_dtype) != LBT_OK) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  lbt::Layout L{};
+  lbt::make_layout(ar, L, n_rows, n_features, n_outputs, max_depth, split_samples,
+                   x_dtype == LBT_F64 ? 8 : 4, hist_cache_bytes);
+  return ar.used + 256;
+}
+
+int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
+                   int64_t n_rows, int32_t n_features, const double* g, const double* h,
+                   int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
+                   double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
+                   void* workspace, size_t workspace_bytes, lbt_build_taps* taps)
+{
+  LBT_TRY(lbt::validate(n_rows, n_features, n_outputs, params, x_dtype));
+  LBT_REQUIRE(X && g && h && leaf && feature && split && gain && hessian, "null input or output pointer");
+  LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
+  if (workspace == nullptr) {
+    lbt::set_error("workspace is null; size it with lbt_build_tree_workspace_bytes");
+    return LBT_ERR_WORKSPACE;
+  }
+  lbt::Arena ar;
+  uintptr_t raw     = reinterpret_cast<uintptr_t>(workspace);
+  uintptr_t aligned = (raw + 255) & ~uintptr_t(255);
+  ar.base           = reinterpret_cast<char*>(aligned);
+  ar.cap            = workspace_bytes > (aligned - raw) ? workspace_bytes - (aligned - raw) : 0;
+  lbt::Layout L{};
+  lbt::make_layout(ar, L, n_rows, n_features, n_outputs, params->max_depth, params->split_samples,
+                   x_dtype == LBT_F64 ? 8 : 4, params->hist_cache_bytes);
+  if (ar.failed) {
+    lbt::set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int rc;
+  if (x_dtype == LBT_F32)
+    rc = lbt::build_tree_impl<float>(s, static_cast<const float*>(X), row_offset, n_rows, n_features, g, h,
+                                     n_outputs, feature_set, *params, leaf, feature, split, gain, hessian, L, taps);
+  else
+    rc = lbt::build_tree_impl<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, g, h,
+                                      n_outputs, feature_set, *params, leaf, feature, split, gain, hessian, L, taps);
+  if (rc != LBT_OK && lbt::profiler().enabled) {
+    (void)hipStreamSynchronize(s);
+    lbt::profiler().collect();
+  }
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,83 @@
+// Error reporting, version and the event-based profiler of liblbtree.so.
+#include "lbt_internal.h"
+
+#include <cstring>
+
+namespace lbt {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...)
+{
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+Profiler& profiler()
+{
+  static Profiler p;
+  return p;
+}
+
+void Profiler::begin(int cls, int level, double bytes, hipStream_t s)
+{
+  ProfSpan sp{};
+  sp.cls   = cls;
+  sp.level = level;
+  sp.bytes = bytes;
+  if (hipEventCreate(&sp.start) != hipSuccess || hipEventCreate(&sp.stop) != hipSuccess) return;
+  (void)hipEventRecord(sp.start, s);
+  open.push_back(sp);
+}
+
+void Profiler::end(hipStream_t s)
+{
+  if (open.empty()) return;
+  (void)hipEventRecord(open.back().stop, s);
+}
+
+void Profiler::collect()
+{
+  for (auto& sp : open) {
+    float ms = 0.f;
+    if (hipEventSynchronize(sp.stop) == hipSuccess &&
+        hipEventElapsedTime(&ms, sp.start, sp.stop) == hipSuccess) {
+      acc.launches[sp.cls] += 1;
+      acc.ms[sp.cls] += ms;
+      acc.bytes[sp.cls] += sp.bytes;
+      if (sp.cls == LBT_PROF_HISTOGRAM && sp.level >= 0 && sp.level < 64) {
+        if (sp.level + 1 > acc.n_levels) acc.n_levels = sp.level + 1;
+        acc.level_ms[sp.level] += ms;
+        acc.level_bytes[sp.level] += sp.bytes;
+      }
+    }
+    (void)hipEventDestroy(sp.start);
+    (void)hipEventDestroy(sp.stop);
+  }
+  open.clear();
+}
+
+}  // namespace lbt
+
+extern "C" {
+
+const char* lbt_last_error(void) { return lbt::g_error; }
+
+int lbt_version(void) { return 1; }
+
+void lbt_profile_enable(int on) { lbt::profiler().enabled = on != 0; }
+
+void lbt_profile_reset(void)
+{
+  auto& p = lbt::profiler();
+  std::memset(&p.acc, 0, sizeof(p.acc));
+}
+
+void lbt_profile_get(lbt_profile* out)
+{
+  if (out) *out = lbt::profiler().acc;
+}
+
+}  // extern "C"

@@ -1,0 +1,219 @@
+// Internal declarations shared by the translation units of liblbtree.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "../../include/lbtree.h"
+
+namespace lbt {
+
+// ---------------------------------------------------------------- errors
+
+void set_error(const char* fmt, ...);
+
+#define LBT_HIP(call)                                                                  \
+  do {                                                                                 \
+    hipError_t e__ = (call);                                                           \
+    if (e__ != hipSuccess) {                                                           \
+      ::lbt::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__, \
+                       __LINE__);                                                      \
+      return LBT_ERR_HIP;                                                              \
+    }                                                                                  \
+  } while (0)
+
+#define LBT_REQUIRE(cond, ...)          \
+  do {                                  \
+    if (!(cond)) {                      \
+      ::lbt::set_error(__VA_ARGS__);    \
+      return LBT_ERR_INVALID;           \
+    }                                   \
+  } while (0)
+
+#define LBT_TRY(expr)            \
+  do {                           \
+    int rc__ = (expr);           \
+    if (rc__ != LBT_OK) return rc__; \
+  } while (0)
+
+// ---------------------------------------------------------------- workspace
+
+// Bump allocator over the caller's scratch buffer. In "measure" mode it only
+// adds up sizes, so the same code path computes lbt_*_workspace_bytes.
+struct Arena {
+  char* base   = nullptr;
+  size_t cap   = 0;
+  size_t used  = 0;
+  bool measure = false;
+  bool failed  = false;
+
+  template <typename T>
+  T* take(size_t n)
+  {
+    size_t bytes = (n * sizeof(T) + 255) & ~size_t(255);
+    size_t at    = used;
+    used += bytes;
+    if (measure) return nullptr;
+    if (used > cap) {
+      failed = true;
+      return nullptr;
+    }
+    return reinterpret_cast<T*>(base + at);
+  }
+};
+
+// ---------------------------------------------------------------- profiling
+
+struct ProfSpan {
+  int cls;
+  int level;  // tree level for histogram spans, else -1
+  double bytes;
+  hipEvent_t start, stop;
+};
+
+struct Profiler {
+  bool enabled = false;
+  lbt_profile acc{};
+  std::vector<ProfSpan> open;  // spans of the call in flight
+  void begin(int cls, int level, double bytes, hipStream_t s);
+  void end(hipStream_t s);
+  void collect();  // after the stream has been synchronised
+};
+Profiler& profiler();
+
+struct ProfScope {
+  hipStream_t s;
+  bool on;
+  ProfScope(int cls, hipStream_t stream, double bytes = 0.0, int level = -1) : s(stream)
+  {
+    on = profiler().enabled;
+    if (on) profiler().begin(cls, level, bytes, s);
+  }
+  ~ProfScope()
+  {
+    if (on) profiler().end(s);
+  }
+};
+
+// ---------------------------------------------------------------- device math
+
+#define LBT_M 2147483647u
+#define LBT_A 48271u
+
+// thrust::minstd_rand seeding: s mod m, 1 if that is 0.
+__host__ __device__ inline uint32_t minstd_seed(uint32_t s)
+{
+  uint32_t x = s % LBT_M;
+  return x == 0 ? 1u : x;
+}
+__host__ __device__ inline uint32_t minstd_next(uint32_t x)
+{
+  return static_cast<uint32_t>((static_cast<uint64_t>(x) * LBT_A) % LBT_M);
+}
+__host__ __device__ inline uint32_t minstd_discard(uint32_t x, uint64_t z)
+{
+  uint64_t mult = LBT_A, acc = 1;
+  while (z > 0) {
+    if (z & 1) acc = (acc * mult) % LBT_M;
+    mult = (mult * mult) % LBT_M;
+    z >>= 1;
+  }
+  return static_cast<uint32_t>((static_cast<uint64_t>(x) * acc) % LBT_M);
+}
+// thrust::uniform_real_distribution<double>(0,1) on one raw draw.
+__host__ __device__ inline double uniform01(uint32_t draw)
+{
+  return static_cast<double>(draw - 1u) / 2147483646.0;
+}
+
+// fmix64 on a signed 64-bit value: arithmetic right shifts, wrapping multiplies
+// (reference: build_tree.cu:143-154).
+__host__ __device__ inline int64_t hash64(int64_t k)
+{
+  k ^= k >> 33;
+  k = static_cast<int64_t>(static_cast<uint64_t>(k) * 0xff51afd7ed558ccdULL);
+  k ^= k >> 33;
+  k = static_cast<int64_t>(static_cast<uint64_t>(k) * 0xc4ceb9fe1a85ec53ULL);
+  k ^= k >> 33;
+  return k;
+}
+__host__ __device__ inline int64_t hash_combine1(int64_t seed, int64_t v)
+{
+  uint64_t sum = static_cast<uint64_t>(hash64(v)) + 0x9e3779b9ULL +
+                 (static_cast<uint64_t>(seed) << 6) + static_cast<uint64_t>(seed >> 2);
+  return seed ^ static_cast<int64_t>(sum);
+}
+// seed of the stochastic rounding of (row, output): build_tree.cu:190, :353
+__host__ __device__ inline int64_t gpair_seed(int64_t seed, int64_t row, int64_t output)
+{
+  return hash_combine1(hash_combine1(seed, row), output);
+}
+
+// build_tree.h:106-121
+__host__ __device__ inline double leaf_gain(double grad, double hess, double l1, double reg)
+{
+  double z = 0.0;
+  if (grad > l1) {
+    z = grad - l1;
+  } else if (grad < -l1) {
+    z = grad + l1;
+  }
+  return (z * z) / (hess + reg);
+}
+// build_tree.h:123-137
+__host__ __device__ inline double calculate_gain(double gl, double hl, double gr, double hr,
+                                                 double gp, double hp, double l1, double reg,
+                                                 double min_split_gain)
+{
+  return (0.5 * (leaf_gain(gl, hl, l1, reg) + leaf_gain(gr, hr, l1, reg) -
+                 leaf_gain(gp, hp, l1, reg))) -
+         min_split_gain;
+}
+// build_tree.h:139-152
+__host__ __device__ inline double calculate_leaf_value(double G, double H, double l1, double l2)
+{
+  double z = 0.0;
+  if (G > l1) {
+    z = G - l1;
+  } else if (G < -l1) {
+    z = G + l1;
+  }
+  return -z / (H + l2);
+}
+
+// build_tree.h:64-74
+__host__ __device__ inline int parent_of(int i) { return (i - 1) / 2; }
+__host__ __device__ inline int left_child(int i) { return 2 * i + 1; }
+__host__ __device__ inline int right_child(int i) { return 2 * i + 2; }
+__host__ __device__ inline int sibling_of(int i) { return (i % 2 == 0) ? i - 1 : i + 1; }
+inline int64_t level_begin(int l) { return (int64_t(1) << l) - 1; }
+inline int64_t level_end(int l) { return (int64_t(1) << (l + 1)) - 1; }
+
+struct I64Pair {
+  int64_t grad;
+  int64_t hess;
+};
+
+// build_tree.h:76-104; node_sums is [max_nodes][K] pairs, output 0 decides.
+__device__ inline bool compute_histogram_bin(int node, const I64Pair* node_sums, int K,
+                                             bool parent_histogram_exists)
+{
+  if (node == 0) return true;
+  if (node < 0) return false;
+  if (!parent_histogram_exists) return true;
+  int parent = parent_of(node);
+  int l = left_child(parent), r = right_child(parent);
+  int64_t hl = node_sums[static_cast<int64_t>(l) * K].hess;
+  int64_t hr = node_sums[static_cast<int64_t>(r) * K].hess;
+  int histogram_node = (hl < hr) ? l : r;
+  return histogram_node == node;
+}
+
+inline int ceil_div(int64_t a, int64_t b) { return static_cast<int>((a + b - 1) / b); }
+
+}  // namespace lbt

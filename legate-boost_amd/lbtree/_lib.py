@@ -1,0 +1,130 @@
+"""ctypes binding of liblbtree.so (the C ABI declared in include/lbtree.h).
+
+The library is the only compute path: if it has not been built the import
+fails, there is no fallback.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "liblbtree.so")
+
+LBT_OK = 0
+LBT_F32 = 0
+LBT_F64 = 1
+LBT_MAX_SPLIT_SAMPLES = 2048
+PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "positions", "other", "predict"]
+
+
+class BuildParams(C.Structure):
+    _fields_ = [
+        ("max_depth", C.c_int32),
+        ("max_nodes", C.c_int32),
+        ("split_samples", C.c_int32),
+        ("seed", C.c_int32),
+        ("dataset_rows", C.c_int64),
+        ("l1_regularization", C.c_double),
+        ("l2_regularization", C.c_double),
+        ("min_split_gain", C.c_double),
+        ("hist_cache_bytes", C.c_int64),
+    ]
+
+
+class BuildTaps(C.Structure):
+    _fields_ = [
+        ("proposals", C.c_void_p),
+        ("row_pointers", C.c_void_p),
+        ("quantised", C.c_void_p),
+        ("node_sums", C.c_void_p),
+        ("positions", C.c_void_p),
+        ("positions_per_level", C.c_void_p),
+        ("histogram", C.c_void_p),
+        ("histogram_capacity", C.c_int64),
+        ("n_bins", C.c_int32),
+        ("hist_node_begin", C.c_int32),
+        ("hist_node_end", C.c_int32),
+        ("scales", C.c_double * 4),
+        ("level_instances", C.c_void_p),
+        ("level_built_instances", C.c_void_p),
+        ("level_built_nodes", C.c_void_p),
+    ]
+
+
+class Profile(C.Structure):
+    _fields_ = [
+        ("launches", C.c_int64 * 8),
+        ("ms", C.c_double * 8),
+        ("bytes", C.c_double * 8),
+        ("n_levels", C.c_int32),
+        ("level_ms", C.c_double * 64),
+        ("level_bytes", C.c_double * 64),
+    ]
+
+
+class LbtError(RuntimeError):
+    """Raised for a non-zero status; the reference throws std::runtime_error at the same places."""
+
+
+def _load():
+    if not os.path.exists(SO_PATH):
+        raise ImportError(
+            "liblbtree.so is missing (%s): build it with `make -C legate-boost_amd/csrc` "
+            "or __graft_entry__.build(); there is no fallback path" % SO_PATH
+        )
+    lib = C.CDLL(SO_PATH)
+    lib.lbt_last_error.restype = C.c_char_p
+    lib.lbt_version.restype = C.c_int
+    lib.lbt_build_tree_workspace_bytes.restype = C.c_size_t
+    lib.lbt_build_tree_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
+                                                   C.c_int64]
+    lib.lbt_build_tree.restype = C.c_int
+    lib.lbt_build_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_void_p,
+                                   C.c_void_p, C.c_int32, C.c_void_p, C.POINTER(BuildParams), C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(BuildTaps)]
+    lib.lbt_predict.restype = C.c_int
+    lib.lbt_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_void_p,
+                                C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+    lib.lbt_update_tree_workspace_bytes.restype = C.c_size_t
+    lib.lbt_update_tree_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
+    lib.lbt_update_tree.restype = C.c_int
+    lib.lbt_update_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p,
+                                    C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_double, C.c_void_p,
+                                    C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_profile_enable.restype = None
+    lib.lbt_profile_enable.argtypes = [C.c_int]
+    lib.lbt_profile_reset.restype = None
+    lib.lbt_profile_get.restype = None
+    lib.lbt_profile_get.argtypes = [C.POINTER(Profile)]
+    return lib
+
+
+lib = _load()
+
+EXPORTS = [
+    "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_predict",
+    "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_profile_enable", "lbt_profile_reset",
+    "lbt_profile_get",
+]
+
+
+def check(rc):
+    if rc != LBT_OK:
+        raise LbtError("lbtree status %d: %s" % (rc, lib.lbt_last_error().decode()))
+
+
+def profile_enable(on=True):
+    lib.lbt_profile_enable(1 if on else 0)
+
+
+def profile_reset():
+    lib.lbt_profile_reset()
+
+
+def profile_get():
+    p = Profile()
+    lib.lbt_profile_get(C.byref(p))
+    out = {}
+    for i, name in enumerate(PROF_CLASSES):
+        out[name] = {"launches": p.launches[i], "ms": p.ms[i], "bytes": p.bytes[i]}
+    out["levels"] = [{"ms": p.level_ms[d], "bytes": p.level_bytes[d]} for d in range(p.n_levels)]
+    return out

@@ -1,0 +1,84 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports
+every symbol that include/lbtree.h declares, and rejects bad arguments before
+touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "lbtree.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lbt_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from lbtree import _lib
+
+    names = declared_symbols()
+    assert "lbt_build_tree" in names and "lbt_predict" in names and "lbt_update_tree" in names
+    for n in names:
+        assert hasattr(_lib.lib, n), n
+    assert sorted(_lib.EXPORTS) == names
+    assert _lib.lib.lbt_version() >= 1
+
+
+def test_workspace_query():
+    from lbtree import _lib
+
+    q = _lib.lib.lbt_build_tree_workspace_bytes
+    a = q(100000, 32, 1, 6, 256, _lib.LBT_F32, 0)
+    b = q(200000, 32, 1, 6, 256, _lib.LBT_F32, 0)
+    c = q(100000, 32, 4, 6, 256, _lib.LBT_F32, 0)
+    assert 0 < a < b and a < c
+    # config 2 of the benchmark fits comfortably next to a 4 GB X
+    assert q(10_000_000, 100, 1, 8, 256, _lib.LBT_F32, 0) < 1_000_000_000
+    # invalid shapes give 0
+    assert q(0, 32, 1, 6, 256, _lib.LBT_F32, 0) == 0
+    assert q(1000, 32, 1, 6, 4096, _lib.LBT_F32, 0) == 0
+    assert q(1000, 32, 1, 40, 256, _lib.LBT_F32, 0) == 0
+    assert q(1000, 32, 1, 6, 256, 7, 0) == 0
+    assert _lib.lib.lbt_update_tree_workspace_bytes(1000, 2, 127) >= 127 * 2 * 16
+
+
+def test_bad_arguments_are_rejected_without_a_gpu():
+    from lbtree import _lib
+
+    prm = _lib.BuildParams(3, 15, 16, 0, 10, 0.0, 1.0, 0.0, 0)
+    one = C.c_void_p(16)  # never dereferenced: validation fails first
+    rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
+                                 one, one, None, 0, None)
+    assert rc == -3 and b"workspace" in _lib.lib.lbt_last_error()
+    prm.max_nodes = 14
+    rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
+                                 one, one, one, 1 << 20, None)
+    assert rc == -1 and b"max_nodes" in _lib.lib.lbt_last_error()
+    prm.max_nodes = 15
+    prm.split_samples = 4096
+    rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
+                                 one, one, one, 1 << 20, None)
+    assert rc == -1 and b"split_samples" in _lib.lib.lbt_last_error()
+    rc = _lib.lib.lbt_build_tree(None, one, 5, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one, one, one,
+                                 one, 1 << 20, None)
+    assert rc == -1
+    rc = _lib.lib.lbt_predict(None, one, 9, 10, 2, 0, None, None, None, None, 1, one)
+    assert rc == -1
+    with pytest.raises(_lib.LbtError):
+        _lib.check(rc)
+
+
+def test_tree_constructor_mirrors_reference_checks():
+    from lbtree.models import Tree
+
+    with pytest.raises(ValueError, match="split_samples must be <= 2048"):
+        Tree(split_samples=4096)
+    with pytest.warns(FutureWarning):
+        t = Tree(alpha=3.0)
+    assert t.l2_regularization == 3.0
+    t = Tree()
+    assert (t.max_depth, t.split_samples, t.feature_fraction, t.l1_regularization, t.l2_regularization,
+            t.min_split_gain) == (8, 256, 1.0, 0.0, 1.0, 0.0)

@@ -1,0 +1,204 @@
+"""GPU parity: liblbtree.so (through the C ABI) against the CPU oracle on the
+same seeded inputs. Integer results (quantised gradients, histograms, node
+sums, splits, positions) must be bit-exact; leaf values are additionally
+checked against the 1e-6 relative tolerance, predictions against 1e-5 absolute."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(seed, n, f, k, dtype=np.float32, lowcard=True):
+    rs = np.random.RandomState(seed)
+    X = rs.randn(n, f).astype(dtype)
+    if lowcard and f > 2:
+        X[:, 1] = rs.randint(0, 4, n)
+        X[:, 2] = 0.25
+    g = rs.randn(n, k)
+    h = rs.rand(n, k) + 0.1
+    return X, g, h
+
+
+@pytest.mark.parametrize("n,f,k,depth,s,dtype", [
+    (1000, 4, 1, 3, 16, np.float32),
+    (5000, 10, 1, 5, 64, np.float32),
+    (5000, 10, 3, 4, 64, np.float64),
+    (20000, 33, 2, 6, 256, np.float32),
+    (3000, 7, 1, 8, 2048, np.float32),
+    (2, 1, 1, 1, 256, np.float64),
+    (1, 3, 2, 2, 8, np.float32),
+    (700, 300, 1, 3, 5, np.float32),
+])
+def test_build_tree_bit_exact(n, f, k, depth, s, dtype):
+    import gpu_util as gu
+
+    X, g, h = _problem(n * 7 + f, n, f, k, dtype)
+    gr, cr = gu.both(X, g, h, levels=True, max_depth=depth, split_samples=s, seed=12345)
+    gu.assert_tree_parity(gr, cr, levels=True)
+
+
+def test_depth_zero_and_regularisation_variants():
+    import gpu_util as gu
+
+    X, g, h = _problem(5, 4000, 6, 2)
+    for kw in [dict(max_depth=0, split_samples=16, seed=1),
+               dict(max_depth=4, split_samples=32, seed=2, l1_regularization=0.7, l2_regularization=0.0),
+               dict(max_depth=4, split_samples=32, seed=3, l2_regularization=5.0, min_split_gain=0.05),
+               dict(max_depth=5, split_samples=32, seed=2**31 - 1)]:
+        gr, cr = gu.both(X, g, h, **kw)
+        gu.assert_tree_parity(gr, cr)
+
+
+def test_feature_set():
+    import gpu_util as gu
+
+    X, g, h = _problem(6, 3000, 8, 1)
+    fs = np.array([0, 1, 0, 0, 1, 0, 0, 1], bool)
+    gr, cr = gu.both(X, g, h, max_depth=5, split_samples=32, seed=4, feature_set=fs)
+    gu.assert_tree_parity(gr, cr)
+    used = set(gu.cpu(gr.feature)[gu.cpu(gr.feature) >= 0].tolist())
+    assert used and used <= {1, 4, 7}
+
+
+def test_small_histogram_budget_batches():
+    import gpu_util as gu
+
+    X, g, h = _problem(8, 3000, 5, 2)
+    ref = None
+    for budget in [0, 40000, 6000, 1]:
+        gr, cr = gu.both(X, g, h, max_depth=5, split_samples=16, seed=9, hist_cache_bytes=budget)
+        gu.assert_tree_parity(gr, cr)
+        if ref is None:
+            ref = gu.cpu(gr.feature).copy()
+        assert np.array_equal(gu.cpu(gr.feature), ref)
+
+
+def test_deep_tree_with_duplicates_and_small_nodes():
+    import gpu_util as gu
+
+    rs = np.random.RandomState(3)
+    n, f = 6000, 12
+    X = np.exp(rs.randn(n, f) * 1.5).astype(np.float32)
+    X[:, :4] = rs.randint(0, 16, (n, 4))
+    y = (X[:, 0] > 7).astype(float) + (X[:, 5] > 1.0) * 2.0 + rs.randn(n) * 0.2
+    g = (0.0 - y).reshape(-1, 1)
+    h = np.ones((n, 1))
+    gr, cr = gu.both(X, g, h, levels=True, max_depth=12, split_samples=512, seed=77)
+    gu.assert_tree_parity(gr, cr, levels=True)
+    assert (cr.feature != -1).sum() > 100
+
+
+def test_tie_rule_on_gpu():
+    import gpu_util as gu
+
+    n = 64
+    Xp = np.arange(1, 601, dtype=np.float32).reshape(-1, 1)
+    X = np.zeros((n, 1), np.float32)
+    X[: n // 2, 0] = 470.0
+    X[n // 2:, 0] = 600.0
+    Xall = np.concatenate([Xp, X])
+    g = np.zeros((len(Xall), 1))
+    h = np.full((len(Xall), 1), 1e-300)
+    g[600: 600 + n // 2] = -1.0
+    g[600 + n // 2:] = 1.0
+    h[600:] = 1.0
+    gr, cr = gu.both(Xall, g, h, max_depth=1, split_samples=2048, seed=0)
+    gu.assert_tree_parity(gr, cr)
+    bin_idx = int(np.searchsorted(cr.proposals, np.float32(gu.cpu(gr.split_value)[0])))
+    assert bin_idx == 511
+
+
+def test_config1_boosting_rounds_match_oracle_round_by_round():
+    """BASELINE config 1: 100000x32, squared error, depth 6, 10 rounds, lr 0.1.
+    Each round's task inputs (X, g, h, seed) go to both implementations."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(0)
+    n, f = 100000, 32
+    X = rs.random_sample((n, f)).astype(np.float32)
+    y = np.sin(2 * np.pi * X[:, :4].astype(np.float64)).sum(axis=1) + rs.normal(0, 0.1, n)
+    Xd = ops.as_device(X)
+    est_rs = np.random.RandomState(0)
+    pred = np.full((n, 1), y.mean())
+    losses = []
+    for rnd in range(10):
+        g = (pred - y.reshape(-1, 1)) * 0.1
+        h = np.ones((n, 1))
+        seed = int(est_rs.randint(0, 2**31))
+        gr, cr = gu.both(Xd if False else X, g, h, max_depth=6, split_samples=256, seed=seed)
+        gu.assert_tree_parity(gr, cr)
+        p_gpu = gu.cpu(ops.predict(Xd, [(gr.leaf_value, gr.feature, gr.split_value)], 1))
+        p_cpu = orc.predict(X, [(cr.leaf_value, cr.feature, cr.split_value)], 1)
+        assert np.abs(p_gpu - p_cpu).max() <= 1e-5
+        assert np.array_equal(p_gpu, p_cpu)
+        pred = pred + p_cpu
+        losses.append(((pred[:, 0] - y) ** 2).mean())
+    assert all(b < a for a, b in zip(losses, losses[1:]))
+
+
+def test_predict_matches_oracle_multi_tree_multi_output():
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(21)
+    X = rs.randn(30000, 16).astype(np.float32)
+    trees_c, trees_g = [], []
+    for t in range(130):  # more than one launch batch
+        m = 2 ** 5 - 1
+        feat = -np.ones(m, np.int32)
+        feat[: 2 ** 4 - 1] = rs.randint(0, 16, 2 ** 4 - 1)
+        # some early leaves
+        feat[rs.randint(1, 15, 2)] = -1
+        split = rs.randn(m)
+        leaf = rs.randn(m, 3) * 0.01
+        trees_c.append((leaf, feat, split))
+        trees_g.append((ops.as_device(leaf), ops.as_device(feat), ops.as_device(split)))
+    want = orc.predict(X, trees_c, 3)
+    got = gu.cpu(ops.predict(X, trees_g, 3))
+    assert np.array_equal(got, want)
+    X64 = X.astype(np.float64)
+    got64 = gu.cpu(ops.predict(X64, trees_g[:3], 3))
+    assert np.array_equal(got64, orc.predict(X64, trees_c[:3], 3))
+    assert np.array_equal(gu.cpu(ops.predict(X, [], 3)), np.zeros((30000, 3)))
+
+
+def test_update_tree_matches_oracle_within_rounding():
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    X, g, h = _problem(31, 20000, 6, 2)
+    gr, cr = gu.both(X, g, h, max_depth=5, split_samples=64, seed=8)
+    leaf_c, hess_c = orc.update_tree(X, g, h, cr.feature, cr.split_value, 0.3, 1.0)
+    leaf_g, hess_g = ops.update_tree(X, g, h, gr.feature, gr.split_value, 0.3, 1.0)
+    # double sums in a different order: 1e-6 relative, as the task states for leaf values
+    assert np.allclose(gu.cpu(leaf_g), leaf_c, rtol=1e-6, atol=1e-12)
+    assert np.allclose(gu.cpu(hess_g), hess_c, rtol=1e-9)
+
+
+def test_two_runs_are_bit_identical():
+    import gpu_util as gu
+
+    X, g, h = _problem(2, 50000, 20, 1)
+    a = gu.gpu_build(X, g, h, max_depth=6, split_samples=256, seed=5)
+    b = gu.gpu_build(X, g, h, max_depth=6, split_samples=256, seed=5)
+    torch.cuda.synchronize()
+    for name in ["leaf_value", "feature", "split_value", "gain", "hessian", "positions", "histogram"]:
+        assert torch.equal(getattr(a, name), getattr(b, name)), name
+
+
+def test_errors_surface_as_exceptions():
+    from lbtree import _lib, ops
+
+    X = np.zeros((10, 2), np.float32)
+    g = np.zeros((10, 1))
+    with pytest.raises(_lib.LbtError):
+        ops.build_tree(X, g, g, max_depth=2, split_samples=4096, seed=0)
+    with pytest.raises(_lib.LbtError):
+        ops.build_tree(X.astype(np.float16), g, g, max_depth=2, split_samples=16, seed=0)
+    with pytest.raises(_lib.LbtError):
+        ops.build_tree(X, g[:5], g[:5], max_depth=2, split_samples=16, seed=0)
