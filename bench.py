@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the tree-learner path on one MI355X.
+
+Default workload: BASELINE config 2 -- LBRegressor squared error,
+Tree(max_depth=8, split_samples=256), X 10,000,000 x 100 f32. One step is one
+boosting round: gradient step, BuildTreeTask, PredictTask of the new tree and
+the prediction update, all with inputs resident in HBM.
+
+Prints ONE JSON line. `roofline` describes the histogram kernel (HIP events on
+the stream of the call, summed over the timed rounds); `cpu_baseline` is the
+restated CPU variant of the reference timed on the host cores of this machine
+on a row sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "legate-boost_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--rows", type=int, default=0, help="override the number of rows (0 = the configuration's)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    return ap.parse_args()
+
+
+def cpu_baseline_build(X_sample, y_sample, max_depth, split_samples, lr, full_rows, seconds, n_outputs_classes=0):
+    """Rounds/s of the restated CPU variant on a row sample, scaled to the full row count."""
+    import numpy as np
+
+    import cpu_variant_lib as cv
+
+    cores = max(1, min(16, os.cpu_count() or 1))
+    n = X_sample.shape[0]
+    if n_outputs_classes:
+        k = n_outputs_classes
+        pred = np.zeros((n, k))
+    else:
+        k = 1
+        pred = np.full((n, 1), y_sample.mean())
+    rounds = 0
+    t0 = time.perf_counter()
+    while True:
+        if n_outputs_classes:
+            e = np.exp(pred - pred.max(axis=1, keepdims=True))
+            p = e / e.sum(axis=1, keepdims=True)
+            g = p.copy()
+            g[np.arange(n), y_sample.astype(np.int64)] -= 1.0
+            g *= lr
+            h = np.maximum(p * (1 - p), 1e-8)
+        else:
+            g = (pred - y_sample.reshape(-1, 1)) * lr
+            h = np.ones((n, 1))
+        leaf, feat, split, gain, hess = cv.build_tree(X_sample, g, h, max_depth=max_depth,
+                                                      split_samples=split_samples, seed=rounds, n_threads=cores)
+        pred += cv.predict(X_sample, [(leaf, feat, split)], k, n_threads=cores)
+        rounds += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds and rounds >= 2:
+            break
+    rate_sample = rounds / dt
+    return {
+        "value": rate_sample * n / full_rows,
+        "unit": "rounds/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "first %d of %d rows, %d rounds in %.1f s on %d threads (%.3f rounds/s on the sample, "
+                  "scaled by rows)" % (n, full_rows, rounds, dt, cores, rate_sample),
+    }
+
+
+def bench_training(args):
+    import numpy as np
+    import torch
+
+    from lbtree import _lib, datasets, ops
+
+    cfg = args.config
+    lr = 0.1
+    n_classes = 0
+    if cfg == 1:
+        Xh, yh = datasets.config1()
+        X, y = ops.as_device(Xh), ops.as_device(yh, torch.float64)
+        depth, S, name = 6, 256, "cfg1"
+    elif cfg == 2:
+        rows = args.rows or 10_000_000
+        X, y = datasets.config2(rows, 100)
+        depth, S, name = 8, 256, "cfg2"
+    elif cfg == 3:
+        rows = args.rows or 2_000_000
+        X, y = datasets.config3(rows, 200, 8)
+        depth, S, name, n_classes = 8, 256, "cfg3", 8
+    else:
+        rows = args.rows or 1_000_000
+        X, y = datasets.config4(rows, 50)
+        depth, S, name = 12, 512, "cfg4"
+    n, f = X.shape
+    k = n_classes or 1
+    rs = np.random.RandomState(0)
+    if n_classes:
+        prob = torch.bincount(y.to(torch.int64), minlength=k).to(torch.float64) / n
+        pred = torch.log(prob).reshape(1, -1).repeat(n, 1).contiguous()
+        label = y.to(torch.int64)
+        ar = torch.arange(n, device=X.device)
+    else:
+        pred = torch.full((n, 1), float(y.mean()), dtype=torch.float64, device=X.device)
+        yc = y.reshape(-1, 1)
+
+    def one_round():
+        if n_classes:
+            p = torch.softmax(pred, dim=1)
+            g = p.clone()
+            g[ar, label] -= 1.0
+            g *= lr
+            h = torch.clamp(p * (1.0 - p), min=1e-8)
+        else:
+            g = (pred - yc) * lr
+            h = torch.ones_like(pred)
+        seed = int(rs.randint(0, 2**31))
+        r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
+        pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
+        return r
+
+    def loss():
+        if n_classes:
+            return float(torch.nn.functional.cross_entropy(pred, label))
+        return float(((pred[:, 0] - y) ** 2).mean())
+
+    loss0 = loss()
+    for _ in range(args.warmup):
+        one_round()
+    torch.cuda.synchronize()
+    _lib.profile_reset()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_round()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    _lib.profile_enable(False)
+    prof = _lib.profile_get()
+    loss1 = loss()
+
+    hist = prof["histogram"]
+    achieved = hist["bytes"] / (hist["ms"] * 1e-3) / 1e9 if hist["ms"] > 0 else 0.0
+    levels = [
+        {"level": d, "ms": lv["ms"] / args.steps, "GB": lv["bytes"] / args.steps / 1e9,
+         "GBps": (lv["bytes"] / (lv["ms"] * 1e-3) / 1e9) if lv["ms"] > 0 else 0.0}
+        for d, lv in enumerate(prof["levels"])
+    ]
+    out = {
+        "metric": "boosting rounds/sec + histogram HBM GB/s (% peak), 10M×100 depth 8" if cfg == 2
+        else "boosting rounds/sec + histogram HBM GB/s (% peak), %s" % name,
+        "value": args.steps / dt,
+        "unit": "rounds/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int64",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: %s, Tree(max_depth=%d, split_samples=%d), lr %.1f, X %dx%d f32, K=%d"
+                        % (name, "LBClassifier softmax" if n_classes else "LBRegressor squared error", depth, S, lr,
+                           n, f, k),
+            "rows": n, "features": f, "outputs": k, "max_depth": depth, "split_samples": S,
+            "loss_before": loss0, "loss_after": loss1,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "kernel": "histogram_kernel",
+            "launches": hist["launches"],
+            "avg_launch_ms": hist["ms"] / max(1, hist["launches"]),
+            "bytes_per_round": hist["bytes"] / args.steps,
+            "levels": levels,
+        },
+        "kernel_ms_per_round": {c: prof[c]["ms"] / args.steps for c in _lib.PROF_CLASSES},
+    }
+    if not args.no_cpu_baseline:
+        ns = min(n, 500_000 if cfg != 1 else n)
+        out["cpu_baseline"] = cpu_baseline_build(X[:ns].cpu().numpy(), y[:ns].cpu().numpy(), depth, S, lr, n,
+                                                 args.cpu_seconds, n_classes)
+    return out
+
+
+def bench_predict(args):
+    import numpy as np
+    import torch
+
+    import cpu_variant_lib as cv
+    from lbtree import _lib, datasets, ops
+
+    rows = args.rows or 20_000_000
+    trees = datasets.config5_ensemble()
+    X = datasets.config5_X(rows)
+    for _ in range(max(1, args.warmup)):
+        ops.predict(X, trees, 1)
+    torch.cuda.synchronize()
+    _lib.profile_reset()
+    _lib.profile_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out_t = ops.predict(X, trees, 1)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    _lib.profile_enable(False)
+    byts = rows * (64 * 4 + 8)
+    achieved = byts * args.steps / dt / 1e9
+    out = {
+        "metric": "PredictTask rows/s, 1000 trees depth 8, 20M×64",
+        "value": rows * args.steps / dt,
+        "unit": "rows/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "cfg5: PredictTask, 1000 trees of depth 8, X %dx64 f32, out f64" % rows,
+                   "rows": rows, "trees": 1000, "row_trees_per_s": rows * 1000 * args.steps / dt},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "predict_kernel"},
+    }
+    if not args.no_cpu_baseline:
+        cores = max(1, min(16, os.cpu_count() or 1))
+        ns = 20000
+        Xs = X[:ns].cpu().numpy()
+        th = [(a.cpu().numpy(), b.cpu().numpy(), c.cpu().numpy()) for a, b, c in trees]
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            ref = cv.predict(Xs, th, 1, n_threads=cores)
+            reps += 1
+            if time.perf_counter() - t0 > args.cpu_seconds:
+                break
+        dtc = time.perf_counter() - t0
+        assert np.abs(ref - out_t[:ns].cpu().numpy()).max() <= 1e-5
+        out["cpu_baseline"] = {"value": ns * reps / dtc, "unit": "rows/s", "cores": cores, "kind": "port",
+                               "sample": "first %d rows, all 1000 trees, %d repetitions in %.1f s" % (ns, reps, dtc)}
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives are built)"
+              % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    out = bench_predict(args) if args.config == 5 else bench_training(args)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
