@@ -60,19 +60,6 @@ __device__ inline void atomic_add_i64(int64_t* p, int64_t v)
   atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(v));
 }
 
-struct HistView {
-  I64Pair* data;  // [node - node_begin][K][B]
-  int node_begin;
-  int node_end;
-  int K;
-  int B;
-  __device__ bool contains(int node) const { return node >= node_begin && node < node_end; }
-  __device__ I64Pair* at(int node, int k, int bin) const
-  {
-    return data + ((static_cast<int64_t>(node - node_begin) * K + k) * B + bin);
-  }
-};
-
 // ---------------------------------------------------------------------------
 // tree initialisation / output (build_tree.cu:785-861)
 // ---------------------------------------------------------------------------
@@ -351,242 +338,6 @@ __global__ void fill_positions_kernel(int2* pos, int64_t n)
 {
   int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
   if (i < n) pos[i] = make_int2(0, static_cast<int>(i));
-}
-
-// ---------------------------------------------------------------------------
-// histogram
-// ---------------------------------------------------------------------------
-
-constexpr int kHistThreads  = 512;
-constexpr int kTileRows     = 1024;  // rows of one node handled between two bookkeeping steps
-constexpr int kSmallNodeRows = 64;   // below this a node goes straight to global atomics
-constexpr int kHistUnroll   = 4;
-
-struct LevelMeta {
-  int32_t n_tiles;
-  int32_t pad;
-  long long instances;        // rows in the batch
-  long long built_instances;  // rows whose node's histogram is built
-  long long built_nodes;
-};
-
-// For the nodes [j0, j1) of the current level (level-local indices): decides
-// which are built (build_tree.h:92-104) and cuts their row segments into tiles.
-// tile_start[j - j0] = first tile of node j; tile_start[j1 - j0] = total.
-__global__ void __launch_bounds__(kThreads)
-  plan_tiles_kernel(int j0, int j1, int level_first, const int32_t* seg, const I64Pair* node_sums,
-                    int K, int hist_node_begin, int hist_node_end, int32_t* tile_start,
-                    LevelMeta* meta, LevelMeta* level_total)
-{
-  __shared__ int s_scan[kThreads];
-  __shared__ int s_run;
-  __shared__ unsigned long long s_rb, s_rc, s_nb;
-  if (threadIdx.x == 0) {
-    s_run = 0;
-    s_rb = s_rc = s_nb = 0;
-  }
-  __syncthreads();
-  for (int base = j0; base < j1; base += kThreads) {
-    int j      = base + threadIdx.x;
-    int tiles  = 0;
-    int rows   = 0;
-    bool built = false;
-    if (j < j1) {
-      int node   = level_first + j;
-      rows       = seg[j + 1] - seg[j];
-      int parent = parent_of(node);
-      bool pex   = parent >= hist_node_begin && parent < hist_node_end;
-      built      = compute_histogram_bin(node, node_sums, K, pex);
-      tiles      = built ? (rows + kTileRows - 1) / kTileRows : 0;
-    }
-    s_scan[threadIdx.x] = tiles;
-    __syncthreads();
-    // inclusive scan (Hillis-Steele) over the 256 counts
-    for (int off = 1; off < kThreads; off <<= 1) {
-      int v = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
-      __syncthreads();
-      s_scan[threadIdx.x] += v;
-      __syncthreads();
-    }
-    int run = s_run;
-    if (j < j1) {
-      tile_start[j - j0] = run + s_scan[threadIdx.x] - tiles;
-      atomicAdd(&s_rb, static_cast<unsigned long long>(rows));
-      if (built && rows > 0) {
-        atomicAdd(&s_rc, static_cast<unsigned long long>(rows));
-        atomicAdd(&s_nb, 1ULL);
-      }
-    }
-    __syncthreads();
-    if (threadIdx.x == kThreads - 1) s_run = run + s_scan[kThreads - 1];
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    tile_start[j1 - j0]   = s_run;
-    meta->n_tiles         = s_run;
-    meta->instances       = s_rb;
-    meta->built_instances = s_rc;
-    meta->built_nodes     = s_nb;
-    level_total->instances += s_rb;
-    level_total->built_instances += s_rc;
-    level_total->built_nodes += s_nb;
-  }
-}
-
-template <typename T>
-struct HistArgs {
-  const T* X;
-  int F;
-  const int2* qgh;  // [N][K] packed int32 (grad, hess)
-  int K;
-  const int2* positions;  // (node,row) sorted by node
-  const int32_t* seg;     // level-local segment starts
-  int j0;                 // first level-local node of the batch
-  int n_nodes;            // nodes in the batch
-  int level_first;        // global index of level-local node 0
-  const int32_t* tile_start;
-  const LevelMeta* meta;
-  const T* proposals;
-  const int32_t* row_pointers;
-  const int32_t* groups;  // feature groups: [n_groups+1]
-  int search_steps;       // ceil(log2(max bins of one feature))
-  HistView hist;
-  const unsigned long long* qstats;
-};
-
-// Number of proposals of [p, p+n) that are < x, i.e. lower_bound
-// (build_tree.h:178-185), as a fixed-trip-count branch-free search.
-template <typename T>
-__device__ inline int count_less(const T* p, int n, T x, int steps)
-{
-  int lo = 0;
-  for (int s = 0; s < steps; s++) {
-    int half = n >> 1;
-    bool go  = n > 0 && p[lo + half] < x;
-    lo       = go ? lo + half + 1 : lo;
-    n        = go ? n - half - 1 : half;
-  }
-  return lo;
-}
-
-// One workgroup owns (a contiguous range of row tiles) x (one feature group) x
-// (one output). Thread t is tied to feature f0 + t % gs for its whole life and
-// walks rows t / gs, t / gs + rows_per_pass, ...: the lanes of a wave read
-// consecutive features of a row (contiguous bytes), and the per-feature search
-// range lives in registers. Sums go to an int32 sub-histogram in LDS and are
-// merged into the int64 histogram with global atomics when the node changes
-// (reference: fill_histogram_shared, build_tree.cu:213-480).
-template <typename T>
-__global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
-{
-  extern __shared__ unsigned char smem_raw[];
-  const int group = blockIdx.y;
-  const int k     = blockIdx.z;
-  const int f0 = a.groups[group], f1 = a.groups[group + 1];
-  const int gs   = f1 - f0;
-  const int bin0 = a.row_pointers[f0];
-  const int nb   = a.row_pointers[f1] - bin0;
-  T* s_prop          = reinterpret_cast<T*>(smem_raw);
-  uint32_t* s_hist   = reinterpret_cast<uint32_t*>(smem_raw + ((static_cast<size_t>(nb) * sizeof(T) + 15) & ~size_t(15)));
-
-  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_prop[i] = a.proposals[bin0 + i];
-  for (int i = threadIdx.x; i < 2 * nb; i += kHistThreads) s_hist[i] = 0;
-
-  const int rows_per_pass = kHistThreads / gs;
-  const bool active       = static_cast<int>(threadIdx.x) < rows_per_pass * gs;
-  const int fl            = threadIdx.x % gs;
-  const int rsub          = threadIdx.x / gs;
-  const int f             = f0 + fl;
-  const int pbase         = a.row_pointers[f] - bin0;
-  const int pn            = a.row_pointers[f + 1] - a.row_pointers[f];
-  const unsigned long long max_abs = a.qstats[0];
-
-  const int n_tiles = a.meta->n_tiles;
-  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * blockIdx.x / gridDim.x);
-  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (blockIdx.x + 1) / gridDim.x);
-
-  int cur_node           = -1;
-  unsigned long long acc = 0;  // rows added to the LDS copy since it was last cleared
-  __syncthreads();
-
-  auto flush = [&](int node) {
-    __syncthreads();
-    if (node >= 0) {
-      I64Pair* dst = a.hist.at(node, k, bin0);
-      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
-        int32_t gv  = static_cast<int32_t>(s_hist[2 * i]);
-        uint32_t hv = s_hist[2 * i + 1];
-        if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
-        if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
-        s_hist[2 * i]     = 0;
-        s_hist[2 * i + 1] = 0;
-      }
-    }
-    __syncthreads();
-  };
-
-  for (int tile = t_begin; tile < t_end; tile++) {
-    // node of this tile: last j with tile_start[j] <= tile (uniform over the block)
-    int lo = 0, hi = a.n_nodes;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (a.tile_start[mid] <= tile)
-        lo = mid;
-      else
-        hi = mid - 1;
-    }
-    const int j        = a.j0 + lo;
-    const int node     = a.level_first + j;
-    const int seg_lo   = a.seg[j];
-    const int seg_hi   = a.seg[j + 1];
-    const int r0       = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
-    const int r1       = min(seg_hi, r0 + kTileRows);
-    const int nrows    = r1 - r0;
-    const bool direct  = (seg_hi - seg_lo) < kSmallNodeRows ||
-                        static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
-    if (!direct) {
-      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
-        flush(cur_node);
-        cur_node = node;
-        acc      = 0;
-      }
-      acc += nrows;
-    }
-    if (active) {
-      I64Pair* gdst = a.hist.at(node, k, bin0);
-      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kHistUnroll) {
-        int row[kHistUnroll];
-        T x[kHistUnroll];
-        int2 q[kHistUnroll];
-#pragma unroll
-        for (int u = 0; u < kHistUnroll; u++) {
-          int rr = r + u * rows_per_pass;
-          row[u] = rr < r1 ? a.positions[rr].y : -1;
-        }
-#pragma unroll
-        for (int u = 0; u < kHistUnroll; u++) {
-          if (row[u] >= 0) {
-            x[u] = a.X[static_cast<int64_t>(row[u]) * a.F + f];
-            q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kHistUnroll; u++) {
-          if (row[u] >= 0) {
-            int bin = pbase + count_less(s_prop + pbase, pn, x[u], a.search_steps);
-            if (direct) {
-              atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
-              atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
-            } else {
-              atomicAdd(&s_hist[2 * bin], static_cast<uint32_t>(q[u].x));
-              atomicAdd(&s_hist[2 * bin + 1], static_cast<uint32_t>(q[u].y));
-            }
-          }
-        }
-      }
-    }
-  }
-  flush(cur_node);
 }
 
 // ---------------------------------------------------------------------------
@@ -1014,6 +765,9 @@ struct Layout {
   int32_t* row_pointers;
   int32_t* bin_feature;
   int32_t* groups;
+  uint16_t* tables;
+  void* cell_lo;
+  void* cell_invw;
   // quantiser
   double* part_a[2];
   double* part_b[2];
@@ -1061,6 +815,9 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.row_pointers = ar.take<int32_t>(F + 1);
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
   L.groups       = ar.take<int32_t>(F + 1);
+  L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
+  L.cell_lo      = ar.take<double>(F);
+  L.cell_invw    = ar.take<double>(F);
   int64_t n_chunks = (N * K + 4095) / 4096;
   for (int i = 0; i < 2; i++) {
     L.part_a[i] = ar.take<double>(n_chunks);
@@ -1104,7 +861,6 @@ int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
   return LBT_OK;
 }
 
-constexpr size_t kHistLdsBudget = 64 * 1024;
 
 template <typename T>
 int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F,
@@ -1146,39 +902,14 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
     static_cast<const T*>(L.proposals), B, L.proposals_d);
 
-  // feature groups: consecutive features packed while proposals + int32
-  // sub-histogram fit the LDS budget and the group is not wider than a workgroup
-  std::vector<int32_t> groups{0};
-  int max_feature_bins = 1;
-  size_t lds_bytes     = 0;
-  {
-    const size_t per_bin = sizeof(T) + 8;
-    const int max_bins   = static_cast<int>((kHistLdsBudget - 16) / per_bin);
-    // balance: aim at equal-width groups
-    int64_t n_groups_min = (static_cast<int64_t>(B) + max_bins - 1) / max_bins;
-    int target_bins = static_cast<int>((B + n_groups_min - 1) / n_groups_min);
-    int cur = 0, width = 0;
-    for (int f = 0; f < F; f++) {
-      int nb = rp[f + 1] - rp[f];
-      max_feature_bins = std::max(max_feature_bins, nb);
-      if (width > 0 && (cur + nb > max_bins || width >= kHistThreads / 2 ||
-                        (cur >= target_bins))) {
-        groups.push_back(f);
-        cur   = 0;
-        width = 0;
-      }
-      cur += nb;
-      width++;
-    }
-    groups.push_back(F);
-    int gmax = 0;
-    for (size_t i = 0; i + 1 < groups.size(); i++) gmax = std::max(gmax, rp[groups[i + 1]] - rp[groups[i]]);
-    lds_bytes = ((static_cast<size_t>(gmax) * sizeof(T) + 15) & ~size_t(15)) + static_cast<size_t>(gmax) * 8;
-  }
-  const int n_groups = static_cast<int>(groups.size()) - 1;
-  LBT_HIP(hipMemcpyAsync(L.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
-  int search_steps = 0;
-  while ((1 << search_steps) < max_feature_bins + 1) search_steps++;
+  HistSetup hs;
+  hs.groups     = L.groups;
+  hs.tables     = L.tables;
+  hs.cell_lo    = L.cell_lo;
+  hs.cell_invw  = L.cell_invw;
+  hs.tile_start = L.tile_start;
+  hs.meta       = L.meta;
+  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, rp, L.proposals, L.row_pointers, X));
 
   // ---- quantiser
   {
@@ -1242,13 +973,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     return LBT_ERR_UNSUPPORTED;
   }
 
-  int device = 0, n_cu = 256;
-  LBT_HIP(hipGetDevice(&device));
-  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  if (lds_bytes > 48 * 1024)
-    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(histogram_kernel<T>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-
   int cur_pos = 0, cur_seg = 0;
   const int n_chunks = (B + kSplitChunk - 1) / kSplitChunk;
   for (int depth = 0; depth < max_depth; depth++) {
@@ -1274,24 +998,12 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       }
       const int n_nodes = j1 - j0;
       {
-        ProfScope ps(LBT_PROF_OTHER, stream);
-        plan_tiles_kernel<<<1, kThreads, 0, stream>>>(j0, j1, level_first, L.seg[cur_seg], L.node_sums, K,
-                                                      hv.node_begin, hv.node_end, L.tile_start, L.meta,
-                                                      L.level_totals + depth);
-      }
-      {
-        ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
-        HistArgs<T> a;
-        a.X = X; a.F = F; a.qgh = L.qgh; a.K = K; a.positions = L.pos[cur_pos]; a.seg = L.seg[cur_seg];
-        a.j0 = j0; a.n_nodes = n_nodes; a.level_first = level_first; a.tile_start = L.tile_start;
-        a.meta = L.meta; a.proposals = static_cast<const T*>(L.proposals); a.row_pointers = L.row_pointers;
-        a.groups = L.groups; a.search_steps = search_steps; a.hist = hv; a.qstats = L.qstats;
-        // enough workgroups to fill the device, not more than there can be tiles
-        int64_t max_tiles = (N + kTileRows - 1) / kTileRows + n_nodes;
-        int64_t want      = std::max<int64_t>(1, (static_cast<int64_t>(n_cu) * 4) / (static_cast<int64_t>(n_groups) * K));
-        unsigned gx       = static_cast<unsigned>(std::max<int64_t>(1, std::min(max_tiles, want)));
-        dim3 grid(gx, n_groups, K);
-        histogram_kernel<T><<<grid, kHistThreads, lds_bytes, stream>>>(a);
+        HistBatch hb;
+        hb.X = X; hb.F = F; hb.qgh = L.qgh; hb.K = K; hb.positions = L.pos[cur_pos]; hb.seg = L.seg[cur_seg];
+        hb.j0 = j0; hb.n_nodes = n_nodes; hb.level_first = level_first; hb.proposals = L.proposals;
+        hb.row_pointers = L.row_pointers; hb.hist = hv; hb.qstats = L.qstats; hb.node_sums = L.node_sums;
+        hb.level_total = L.level_totals + depth; hb.n_rows = N;
+        LBT_TRY(hist_launch(stream, hs, hb, depth));
       }
       {
         ProfScope ps(LBT_PROF_SCAN, stream);

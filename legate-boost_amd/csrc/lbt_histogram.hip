@@ -1,0 +1,562 @@
+// Histogram stage of BuildTreeTask: for every row of a node whose histogram is
+// built, every feature f and output k,
+//   hist[node][k][lower_bound(proposals of f, X[row][f])] += quantised (g, h)
+// (rapidsai/legate-boost src/models/tree/build_tree.cu:213-577, build_tree.h:178-185).
+//
+// Layout of the work on gfx950:
+//   * Features are cut into groups whose state fits the LDS of one workgroup
+//     (160 KB): the group's proposals, a packed sub-histogram, and per feature a
+//     direct-lookup table from value to first reachable proposal.
+//   * A workgroup owns (a contiguous range of row tiles) x (group) x (output).
+//     All workgroups are resident at once; those that share a row range sit on
+//     the same XCD so that cache lines straddling two groups are fetched from
+//     HBM once.
+//   * A lane is tied to VEC consecutive features of its group and walks rows, so
+//     the lanes of a wave read consecutive bytes of a row with one 16-byte load
+//     each and keep their features' constants in registers.
+//   * Bin search: cell = clamp((x - lo) * invw) indexes the table, which gives the
+//     number of proposals in cells before it; a short forward probe over the
+//     proposals finishes the search. Any monotone cell function is exact here;
+//     the table is built on the device with the same function.
+//   * (grad, hess) of a row are one 64-bit word (grad in the high half, hess
+//     unsigned in the low half) added with a single LDS atomic; the sub-histogram
+//     is merged into the int64 histogram with global atomics when the workgroup
+//     moves to another node. Before the low half or the signed high half could
+//     overflow (rows * max |q| >= 2^31) the sub-histogram is merged early; rows of
+//     tiny nodes go straight to global atomics.
+#include "lbt_internal.h"
+
+#include <algorithm>
+
+namespace lbt {
+namespace {
+
+constexpr int kPlanThreads   = 256;
+constexpr int kHistThreads   = 1024;
+constexpr int kSmallNodeRows = 64;  // below this a node goes straight to global atomics
+constexpr int kUnroll        = 4;
+constexpr int kLinearProbes  = 4;   // forward probes before falling back to a binary search
+constexpr size_t kLdsBudget  = 160 * 1024 - 512;
+
+// For the nodes [j0, j1) of the current level (level-local indices): decides
+// which are built (build_tree.h:92-104) and cuts their row segments into tiles.
+// tile_start[j - j0] = first tile of node j; tile_start[j1 - j0] = total.
+__global__ void __launch_bounds__(kPlanThreads)
+  plan_tiles_kernel(int j0, int j1, int level_first, const int32_t* seg, const I64Pair* node_sums,
+                    int K, int hist_node_begin, int hist_node_end, int32_t* tile_start,
+                    LevelMeta* meta, LevelMeta* level_total)
+{
+  __shared__ int s_scan[kPlanThreads];
+  __shared__ int s_run;
+  __shared__ unsigned long long s_rb, s_rc, s_nb;
+  if (threadIdx.x == 0) {
+    s_run = 0;
+    s_rb = s_rc = s_nb = 0;
+  }
+  __syncthreads();
+  for (int base = j0; base < j1; base += kPlanThreads) {
+    int j      = base + threadIdx.x;
+    int tiles  = 0;
+    int rows   = 0;
+    bool built = false;
+    if (j < j1) {
+      int node   = level_first + j;
+      rows       = seg[j + 1] - seg[j];
+      int parent = parent_of(node);
+      bool pex   = parent >= hist_node_begin && parent < hist_node_end;
+      built      = compute_histogram_bin(node, node_sums, K, pex);
+      tiles      = built ? (rows + kTileRows - 1) / kTileRows : 0;
+    }
+    s_scan[threadIdx.x] = tiles;
+    __syncthreads();
+    for (int off = 1; off < kPlanThreads; off <<= 1) {
+      int v = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
+      __syncthreads();
+      s_scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    int run = s_run;
+    if (j < j1) {
+      tile_start[j - j0] = run + s_scan[threadIdx.x] - tiles;
+      atomicAdd(&s_rb, static_cast<unsigned long long>(rows));
+      if (built && rows > 0) {
+        atomicAdd(&s_rc, static_cast<unsigned long long>(rows));
+        atomicAdd(&s_nb, 1ULL);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == kPlanThreads - 1) s_run = run + s_scan[kPlanThreads - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    tile_start[j1 - j0]   = s_run;
+    meta->n_tiles         = s_run;
+    meta->instances       = s_rb;
+    meta->built_instances = s_rc;
+    meta->built_nodes     = s_nb;
+    level_total->instances += s_rb;
+    level_total->built_instances += s_rc;
+    level_total->built_nodes += s_nb;
+  }
+}
+
+// The cell of a value: monotone non-decreasing in x for any lo and invw >= 0
+// (rounded subtraction, rounded multiplication by a non-negative constant and
+// clamping are all monotone; NaN goes to cell 0).
+template <typename T>
+__device__ inline int cell_of(T x, T lo, T invw, T cmax)
+{
+  T t = (x - lo) * invw;
+  t   = t > T(0) ? t : T(0);  // false for NaN
+  t   = t < cmax ? t : cmax;
+  return static_cast<int>(t);
+}
+
+// One workgroup per feature. table[c] = number of the feature's proposals
+// whose cell is < c. A value in cell c is >= every proposal in earlier cells
+// and < every proposal in later cells, so its lower bound lies at or after
+// table[c] and is found by probing forward while proposal < x.
+template <typename T>
+__global__ void __launch_bounds__(256)
+  build_cells_kernel(const T* proposals, const int32_t* row_pointers, int C, uint16_t* tables, T* lo_out,
+                     T* invw_out)
+{
+  __shared__ T s_lo, s_invw;
+  const int f = blockIdx.x;
+  const T* p  = proposals + row_pointers[f];
+  const int n = row_pointers[f + 1] - row_pointers[f];
+  if (threadIdx.x == 0) {
+    T lo = T(0), invw = T(0);
+    if (n >= 3) {  // at least two finite proposals (the last one is +inf)
+      lo   = p[0];
+      T hi = p[n - 2];
+      T w  = hi - lo;
+      if (w > T(0) && w < std::numeric_limits<T>::infinity()) {
+        invw = static_cast<T>(C) / w;
+        if (!(invw < std::numeric_limits<T>::infinity())) invw = T(0);
+      }
+      if (!(lo == lo) || lo == -std::numeric_limits<T>::infinity()) {
+        lo   = T(0);
+        invw = T(0);
+      }
+    }
+    s_lo      = lo;
+    s_invw    = invw;
+    lo_out[f]   = lo;
+    invw_out[f] = invw;
+  }
+  __syncthreads();
+  const T lo = s_lo, invw = s_invw, cmax = static_cast<T>(C - 1);
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    // first b with cell(p[b]) >= c
+    int a = 0, len = n;
+    while (len > 0) {
+      int half = len >> 1;
+      if (cell_of(p[a + half], lo, invw, cmax) < c) {
+        a += half + 1;
+        len -= half + 1;
+      } else {
+        len = half;
+      }
+    }
+    // the +inf proposal sits in the last cell, so a <= n - 1 for every c <= C-1
+    tables[static_cast<int64_t>(f) * C + c] = static_cast<uint16_t>(a < n ? a : n - 1);
+  }
+}
+
+template <typename T>
+struct HistArgs {
+  const T* X;
+  int F;
+  const int2* qgh;  // [N][K] packed int32 (grad, hess)
+  int K;
+  const int2* positions;  // (node,row) sorted by node
+  const int32_t* seg;     // level-local segment starts
+  int j0;                 // first level-local node of the batch
+  int n_nodes;            // nodes in the batch
+  int level_first;        // global index of level-local node 0
+  const int32_t* tile_start;
+  const LevelMeta* meta;
+  const T* proposals;
+  const int32_t* row_pointers;
+  const int32_t* groups;  // feature groups: [n_groups+1]
+  const uint16_t* tables;
+  const T* cell_lo;
+  const T* cell_invw;
+  int cells;
+  int search_steps;
+  int n_gk;      // groups * outputs
+  int n_chunks;  // row-tile ranges
+  HistView hist;
+  const unsigned long long* qstats;
+};
+
+template <typename T, int VEC>
+struct VecOf;
+template <>
+struct VecOf<float, 4> {
+  using type = float4;
+};
+template <>
+struct VecOf<float, 2> {
+  using type = float2;
+};
+template <>
+struct VecOf<float, 1> {
+  using type = float;
+};
+template <>
+struct VecOf<double, 2> {
+  using type = double2;
+};
+template <>
+struct VecOf<double, 1> {
+  using type = double;
+};
+
+// Number of proposals in [p, p+n) that are < x (branch-free, fixed trip count).
+template <typename T>
+__device__ inline int count_less(const T* p, int n, T x, int steps)
+{
+  int lo = 0;
+  for (int s = 0; s < steps; s++) {
+    int half = n >> 1;
+    bool go  = n > 0 && p[lo + half] < x;
+    lo       = go ? lo + half + 1 : lo;
+    n        = go ? n - half - 1 : half;
+  }
+  return lo;
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
+{
+  using Vec = typename VecOf<T, VEC>::type;
+  extern __shared__ unsigned char smem_raw[];
+
+  // workgroup -> (row-tile range, group, output). Linear workgroup ids are dealt
+  // round-robin to the 8 XCDs, so id % 8 is the XCD; within an XCD consecutive
+  // slots enumerate (group, output) of one row-tile range.
+  const int xcd   = blockIdx.x & 7;
+  const int slot  = blockIdx.x >> 3;
+  const int gk    = slot % a.n_gk;
+  const int chunk = (slot / a.n_gk) * 8 + xcd;
+  const int group = gk / a.K;
+  const int k     = gk % a.K;
+
+  const int f0 = a.groups[group], f1 = a.groups[group + 1];
+  const int gs   = f1 - f0;
+  const int bin0 = a.row_pointers[f0];
+  const int nb   = a.row_pointers[f1] - bin0;
+  const int C    = a.cells;
+
+  unsigned long long* s_hist = reinterpret_cast<unsigned long long*>(smem_raw);
+  T* s_prop                  = reinterpret_cast<T*>(smem_raw + static_cast<size_t>(nb) * 8);
+  uint16_t* s_cell           = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(nb) * (8 + sizeof(T)));
+
+  for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+    s_prop[i] = a.proposals[bin0 + i];
+    s_hist[i] = 0;
+  }
+  {
+    // tables of the group's features are contiguous: copy as 32-bit words
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(a.tables + static_cast<int64_t>(f0) * C);
+    uint32_t* dst       = reinterpret_cast<uint32_t*>(s_cell);
+    const int words     = gs * C / 2;
+    for (int i = threadIdx.x; i < words; i += kHistThreads) dst[i] = src[i];
+  }
+
+  const int lanes_per_row = (gs + VEC - 1) / VEC;
+  const int rows_per_pass = kHistThreads / lanes_per_row;
+  const int lr            = threadIdx.x % lanes_per_row;
+  const int rsub          = threadIdx.x / lanes_per_row;
+  const bool active       = rsub < rows_per_pass;
+  const int fl            = lr * VEC;  // first group-local feature of this lane
+
+  T c_lo[VEC], c_invw[VEC];
+  int c_cell[VEC], c_prop[VEC], c_end[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; v++) {
+    int f     = min(f0 + fl + v, f1 - 1);
+    c_lo[v]   = a.cell_lo[f];
+    c_invw[v] = a.cell_invw[f];
+    c_cell[v] = (f - f0) * C;
+    c_prop[v] = a.row_pointers[f] - bin0;
+    c_end[v]  = a.row_pointers[f + 1] - bin0;
+  }
+  const T cmax = static_cast<T>(C - 1);
+  const unsigned long long max_abs = a.qstats[0];
+
+  const int n_tiles = a.meta->n_tiles;
+  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / a.n_chunks);
+  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / a.n_chunks);
+
+  int cur_node           = -1;
+  unsigned long long acc = 0;  // rows added to the LDS copy since it was last merged
+  __syncthreads();
+
+  auto flush = [&](int node) {
+    __syncthreads();
+    if (node >= 0) {
+      I64Pair* dst = a.hist.at(node, k, bin0);
+      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+        unsigned long long v = s_hist[i];
+        if (v != 0) {
+          int32_t gv  = static_cast<int32_t>(v >> 32);
+          uint32_t hv = static_cast<uint32_t>(v);
+          if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
+          if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
+          s_hist[i] = 0;
+        }
+      }
+    }
+    __syncthreads();
+  };
+
+  for (int tile = t_begin; tile < t_end; tile++) {
+    // node of this tile: last j with tile_start[j] <= tile (uniform over the workgroup)
+    int lo = 0, hi = a.n_nodes;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (a.tile_start[mid] <= tile)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
+    const int j       = a.j0 + lo;
+    const int node    = a.level_first + j;
+    const int seg_lo  = a.seg[j];
+    const int seg_hi  = a.seg[j + 1];
+    const int r0      = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
+    const int r1      = min(seg_hi, r0 + kTileRows);
+    const int nrows   = r1 - r0;
+    const bool direct = (seg_hi - seg_lo) < kSmallNodeRows ||
+                        static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
+    if (!direct) {
+      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
+        flush(cur_node);
+        cur_node = node;
+        acc      = 0;
+      }
+      acc += nrows;
+    }
+    if (active) {
+      I64Pair* gdst = a.hist.at(node, k, bin0);
+      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kUnroll) {
+        int row[kUnroll];
+        Vec xv[kUnroll];
+        int2 q[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          int rr = r + u * rows_per_pass;
+          row[u] = rr < r1 ? a.positions[rr].y : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          if (row[u] >= 0) {
+            const T* xp = a.X + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
+            if constexpr (VEC == 1)
+              xv[u] = *xp;
+            else
+              xv[u] = *reinterpret_cast<const Vec*>(xp);
+            q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          if (row[u] >= 0) {
+            const unsigned long long packed =
+              (static_cast<unsigned long long>(static_cast<uint32_t>(q[u].x)) << 32) |
+              static_cast<unsigned long long>(static_cast<uint32_t>(q[u].y));
+            T xs[VEC];
+            if constexpr (VEC == 1) {
+              xs[0] = xv[u];
+            } else if constexpr (VEC == 2) {
+              xs[0] = xv[u].x;
+              xs[1] = xv[u].y;
+            } else {
+              xs[0] = xv[u].x;
+              xs[1] = xv[u].y;
+              xs[2] = xv[u].z;
+              xs[3] = xv[u].w;
+            }
+#pragma unroll
+            for (int v = 0; v < VEC; v++) {
+              const T x = xs[v];
+              int bin   = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+              bool lt   = s_prop[bin] < x;
+              int probes = 0;
+              while (__any(lt)) {
+                bin += lt ? 1 : 0;
+                if (++probes == kLinearProbes) {
+                  // crowded cell: finish with a binary search over the rest of the feature
+                  bin += count_less(s_prop + bin, c_end[v] - bin, x, a.search_steps);
+                  break;
+                }
+                lt = s_prop[bin] < x;
+              }
+              if (direct) {
+                atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
+                atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
+              } else {
+                atomicAdd(&s_hist[bin], packed);
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+  flush(cur_node);
+}
+
+template <typename T, int VEC>
+int launch_kernel(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid)
+{
+  static bool attr_set = false;
+  if (!attr_set) {
+    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(histogram_kernel<T, VEC>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBudget)));
+    attr_set = true;
+  }
+  histogram_kernel<T, VEC><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a);
+  return LBT_OK;
+}
+
+template <typename T>
+int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth)
+{
+  {
+    ProfScope ps(LBT_PROF_OTHER, stream);
+    plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
+                                                      b.K, b.hist.node_begin, b.hist.node_end, hs.tile_start,
+                                                      hs.meta, b.level_total);
+  }
+  HistArgs<T> a;
+  a.X = static_cast<const T*>(b.X);
+  a.F = b.F;
+  a.qgh = b.qgh;
+  a.K = b.K;
+  a.positions = b.positions;
+  a.seg = b.seg;
+  a.j0 = b.j0;
+  a.n_nodes = b.n_nodes;
+  a.level_first = b.level_first;
+  a.tile_start = hs.tile_start;
+  a.meta = hs.meta;
+  a.proposals = static_cast<const T*>(b.proposals);
+  a.row_pointers = b.row_pointers;
+  a.groups = hs.groups;
+  a.tables = hs.tables;
+  a.cell_lo = static_cast<const T*>(hs.cell_lo);
+  a.cell_invw = static_cast<const T*>(hs.cell_invw);
+  a.cells = hs.cells;
+  a.search_steps = hs.search_steps;
+  a.hist = b.hist;
+  a.qstats = b.qstats;
+  a.n_gk = hs.n_groups * b.K;
+
+  int device = 0, n_cu = 256;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  // one resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD)
+  const int64_t max_tiles = (b.n_rows + kTileRows - 1) / kTileRows + b.n_nodes;
+  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / a.n_gk);
+  per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
+  a.n_chunks      = static_cast<int>(per_xcd * 8);
+  const unsigned grid = static_cast<unsigned>(per_xcd * 8 * a.n_gk);
+
+  ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
+  if (hs.vec == 4) {
+    if constexpr (sizeof(T) == 4) return launch_kernel<T, 4>(stream, hs, a, grid);
+  }
+  if (hs.vec == 2) return launch_kernel<T, 2>(stream, hs, a, grid);
+  return launch_kernel<T, 1>(stream, hs, a, grid);
+}
+
+}  // namespace
+
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const std::vector<int32_t>& rp,
+                 const void* proposals, const int32_t* row_pointers, const void* X)
+{
+  const size_t elem = is_f64 ? 8 : 4;
+  hs.is_f64         = is_f64;
+  hs.n_features     = F;
+  // widest aligned vector of features a lane can load
+  int vec = is_f64 ? 2 : 4;
+  while (vec > 1 && (F % vec != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0)) vec >>= 1;
+  hs.vec = vec;
+  int max_feature_bins = 1;
+  for (int f = 0; f < F; f++) max_feature_bins = std::max(max_feature_bins, rp[f + 1] - rp[f]);
+  hs.search_steps = 0;
+  while ((1 << hs.search_steps) < max_feature_bins + 1) hs.search_steps++;
+
+  // table size: four cells per proposal of the widest feature, within [64, kMaxCells]
+  int cells = 64;
+  while (cells < 4 * max_feature_bins && cells < kMaxCells) cells <<= 1;
+  std::vector<int32_t> groups;
+  size_t lds = 0;
+  const int max_lanes = kHistThreads / 2;  // at least two rows per pass
+  for (;;) {
+    // bytes of LDS a feature needs: proposals + packed sub-histogram + its table
+    auto chunk_bytes = [&](int f) {
+      size_t bytes = 0;
+      for (int i = f; i < std::min(F, f + vec); i++)
+        bytes += static_cast<size_t>(rp[i + 1] - rp[i]) * (8 + elem) + static_cast<size_t>(cells) * 2;
+      return bytes;
+    };
+    // features are packed in units of `vec`; `target` caps the width of a group
+    auto pack = [&](int target) {
+      groups.assign(1, 0);
+      lds        = 0;
+      size_t cur = 0;
+      int width  = 0;
+      for (int f = 0; f < F; f += vec) {
+        size_t cb = chunk_bytes(f);
+        if (width > 0 && (cur + cb > kLdsBudget || width + vec > target || (width + vec) / vec > max_lanes)) {
+          groups.push_back(f);
+          lds   = std::max(lds, cur);
+          cur   = 0;
+          width = 0;
+        }
+        cur += cb;
+        width += vec;
+      }
+      groups.push_back(F);
+      lds = std::max(lds, cur);
+    };
+    pack(F + vec);  // fewest groups the LDS allows
+    const int n_min = static_cast<int>(groups.size()) - 1;
+    int target      = (F + n_min - 1) / n_min;
+    target          = ((target + vec - 1) / vec) * vec;
+    pack(target);   // same count, balanced widths
+    if (lds <= kLdsBudget) break;
+    if (cells <= 64) {
+      set_error("a feature group does not fit the LDS (%zu bytes)", lds);
+      return LBT_ERR_UNSUPPORTED;
+    }
+    cells >>= 1;
+  }
+  hs.cells     = cells;
+  hs.n_groups  = static_cast<int>(groups.size()) - 1;
+  hs.lds_bytes = (lds + 15) & ~size_t(15);
+  LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
+  ProfScope ps(LBT_PROF_PROPOSALS, stream);
+  if (is_f64)
+    build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,
+                                                     hs.tables, static_cast<double*>(hs.cell_lo),
+                                                     static_cast<double*>(hs.cell_invw));
+  else
+    build_cells_kernel<float><<<F, 256, 0, stream>>>(static_cast<const float*>(proposals), row_pointers, cells,
+                                                    hs.tables, static_cast<float*>(hs.cell_lo),
+                                                    static_cast<float*>(hs.cell_invw));
+  return LBT_OK;
+}
+
+int hist_launch(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth)
+{
+  if (hs.is_f64) return hist_launch_t<double>(stream, hs, b, depth);
+  return hist_launch_t<float>(stream, hs, b, depth);
+}
+
+}  // namespace lbt

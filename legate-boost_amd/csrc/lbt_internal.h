@@ -216,4 +216,84 @@ __device__ inline bool compute_histogram_bin(int node, const I64Pair* node_sums,
 
 inline int ceil_div(int64_t a, int64_t b) { return static_cast<int>((a + b - 1) / b); }
 
+__device__ inline void atomic_add_i64(int64_t* p, int64_t v)
+{
+  atomicAdd(reinterpret_cast<unsigned long long*>(p), static_cast<unsigned long long>(v));
+}
+
+// The histogram buffer: [node - node_begin][K][B] pairs (build_tree.h:231-306).
+struct HistView {
+  I64Pair* data;
+  int node_begin;
+  int node_end;
+  int K;
+  int B;
+  __device__ bool contains(int node) const { return node >= node_begin && node < node_end; }
+  __device__ I64Pair* at(int node, int k, int bin) const
+  {
+    return data + ((static_cast<int64_t>(node - node_begin) * K + k) * B + bin);
+  }
+};
+
+// ---------------------------------------------------------------- histogram stage
+
+// Written by the tile planner for one batch of nodes.
+struct LevelMeta {
+  int32_t n_tiles;
+  int32_t pad;
+  long long instances;        // rows held by the nodes of the batch
+  long long built_instances;  // rows whose node's histogram is built
+  long long built_nodes;
+};
+
+constexpr int kTileRows = 1024;  // rows of one node between two bookkeeping steps
+
+// Per-tree state of the histogram stage: feature groups sized for the LDS of
+// one workgroup and, per feature, a table that maps a value to the first
+// split proposal it can reach (see lbt_histogram.hip).
+struct HistSetup {
+  int n_features     = 0;
+  int n_groups       = 0;
+  int vec            = 1;   // features per lane (1, 2 or 4)
+  int cells          = 0;   // table entries per feature (power of two)
+  int search_steps   = 0;   // ceil(log2(max bins of a feature + 1))
+  size_t lds_bytes   = 0;
+  bool is_f64        = false;
+  // device buffers (carved from the caller's workspace)
+  int32_t* groups    = nullptr;  // [n_groups + 1]
+  uint16_t* tables   = nullptr;  // [n_features][cells]
+  void* cell_lo      = nullptr;  // X dtype [n_features]
+  void* cell_invw    = nullptr;  // X dtype [n_features]
+  int32_t* tile_start = nullptr;
+  LevelMeta* meta    = nullptr;
+};
+
+constexpr int kMaxCells = 2048;
+
+struct HistBatch {
+  const void* X;
+  int F;
+  const int2* qgh;
+  int K;
+  const int2* positions;
+  const int32_t* seg;
+  int j0;
+  int n_nodes;
+  int level_first;
+  const void* proposals;
+  const int32_t* row_pointers;
+  HistView hist;
+  const unsigned long long* qstats;
+  const I64Pair* node_sums;
+  LevelMeta* level_total;
+  int64_t n_rows;
+};
+
+// Chooses groups / table size from the host copy of the row pointers and builds
+// the tables on the device.
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const std::vector<int32_t>& rp,
+                 const void* proposals, const int32_t* row_pointers, const void* X);
+// Plans tiles for the batch and launches the histogram kernel.
+int hist_launch(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth);
+
 }  // namespace lbt
