@@ -765,6 +765,8 @@ struct Layout {
   int32_t* row_pointers;
   int32_t* bin_feature;
   int32_t* groups;
+  int32_t* bgroups;
+  void* binned;
   uint16_t* tables;
   void* cell_lo;
   void* cell_invw;
@@ -815,6 +817,9 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.row_pointers = ar.take<int32_t>(F + 1);
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
   L.groups       = ar.take<int32_t>(F + 1);
+  L.bgroups      = ar.take<int32_t>(F + 1);
+  // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
+  L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(N) * F * (S <= 256 ? 1 : 2) + 16)) : nullptr;
   L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
   L.cell_lo      = ar.take<double>(F);
   L.cell_invw    = ar.take<double>(F);
@@ -908,6 +913,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.cell_lo    = L.cell_lo;
   hs.cell_invw  = L.cell_invw;
   hs.tile_start = L.tile_start;
+  hs.bgroups    = L.bgroups;
+  hs.binned     = L.binned;
   hs.meta       = L.meta;
   LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, rp, L.proposals, L.row_pointers, X));
 
@@ -1087,9 +1094,13 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     // X rows of built nodes + their packed gradients + one position pair per
     // instance + the built histograms written once
     auto& acc = profiler().acc;
+    const bool cached = hs.binned != nullptr;
     for (int d = 0; d < max_depth && d < 64; d++) {
-      double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * sizeof(T) + K * 8.0) +
-                  static_cast<double>(h_levels[d].instances) * 8.0 +
+      // bytes of one feature value as the level reads it (X itself, or its cached bin),
+      // plus the bins the root pass writes
+      double per_value = (cached && d > 0) ? hs.bin_bytes : static_cast<double>(sizeof(T));
+      if (cached && d == 0) per_value += hs.bin_bytes;
+      double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * per_value + K * 8.0 + 8.0) +
                   static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
       acc.level_bytes[d] += by;
       acc.bytes[LBT_PROF_HISTOGRAM] += by;

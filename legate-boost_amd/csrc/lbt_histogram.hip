@@ -189,6 +189,7 @@ struct HistArgs {
   int n_chunks;  // row-tile ranges
   HistView hist;
   const unsigned long long* qstats;
+  void* binned;  // bin cache (written by the root pass, read by the binned kernel)
 };
 
 template <typename T, int VEC>
@@ -228,7 +229,7 @@ __device__ inline int count_less(const T* p, int n, T x, int steps)
   return lo;
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, typename BinT, bool kWriteBins>
 __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
 {
   using Vec = typename VecOf<T, VEC>::type;
@@ -380,6 +381,7 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
               xs[2] = xv[u].z;
               xs[3] = xv[u].w;
             }
+            BinT rel[VEC];
 #pragma unroll
             for (int v = 0; v < VEC; v++) {
               const T x = xs[v];
@@ -395,11 +397,25 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
                 }
                 lt = s_prop[bin] < x;
               }
+              rel[v] = static_cast<BinT>(bin - c_prop[v]);
               if (direct) {
                 atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
                 atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
               } else {
                 atomicAdd(&s_hist[bin], packed);
+              }
+            }
+            if constexpr (kWriteBins) {
+              if (k == 0 && f0 + fl < f1) {
+                BinT* bp = static_cast<BinT*>(a.binned) + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
+                if constexpr (VEC == 4 && sizeof(BinT) == 1) {
+                  *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
+                                                     (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
+                } else {
+#pragma unroll
+                  for (int v = 0; v < VEC; v++)
+                    if (f0 + fl + v < f1) bp[v] = rel[v];
+                }
               }
             }
           }
@@ -410,16 +426,243 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
   flush(cur_node);
 }
 
-template <typename T, int VEC>
-int launch_kernel(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid)
+// Deeper levels: the bins of every (row, feature) are already known, so a lane
+// loads BV cached bins of its row with one load and only accumulates. The
+// sub-histogram is the only LDS state, which allows much wider feature groups.
+template <typename BinT, int BV>
+struct BinVec;
+template <>
+struct BinVec<uint8_t, 4> {
+  using type = uint32_t;
+};
+template <>
+struct BinVec<uint16_t, 4> {
+  using type = uint2;
+};
+template <>
+struct BinVec<uint8_t, 1> {
+  using type = uint8_t;
+};
+template <>
+struct BinVec<uint16_t, 1> {
+  using type = uint16_t;
+};
+
+template <typename BinT, int BV>
+__device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int (&out)[BV])
+{
+  if constexpr (BV == 1) {
+    out[0] = w;
+  } else if constexpr (sizeof(BinT) == 1) {
+    out[0] = w & 0xff;
+    out[1] = (w >> 8) & 0xff;
+    out[2] = (w >> 16) & 0xff;
+    out[3] = w >> 24;
+  } else {
+    out[0] = w.x & 0xffff;
+    out[1] = w.x >> 16;
+    out[2] = w.y & 0xffff;
+    out[3] = w.y >> 16;
+  }
+}
+
+struct BinnedArgs {
+  const void* binned;
+  int F;
+  const int2* qgh;
+  int K;
+  const int2* positions;
+  const int32_t* seg;
+  int j0;
+  int n_nodes;
+  int level_first;
+  const int32_t* tile_start;
+  const LevelMeta* meta;
+  const int32_t* row_pointers;
+  const int32_t* groups;
+  int n_gk;
+  int n_chunks;
+  HistView hist;
+  const unsigned long long* qstats;
+};
+
+template <typename BinT, int BV>
+__global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedArgs a)
+{
+  using Word = typename BinVec<BinT, BV>::type;
+  extern __shared__ unsigned char smem_raw[];
+  const int xcd   = blockIdx.x & 7;
+  const int slot  = blockIdx.x >> 3;
+  const int gk    = slot % a.n_gk;
+  const int chunk = (slot / a.n_gk) * 8 + xcd;
+  const int group = gk / a.K;
+  const int k     = gk % a.K;
+  const int f0 = a.groups[group], f1 = a.groups[group + 1];
+  const int gs   = f1 - f0;
+  const int bin0 = a.row_pointers[f0];
+  const int nb   = a.row_pointers[f1] - bin0;
+  unsigned long long* s_hist = reinterpret_cast<unsigned long long*>(smem_raw);
+  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_hist[i] = 0;
+
+  const int lanes_per_row = (gs + BV - 1) / BV;
+  const int rows_per_pass = kHistThreads / lanes_per_row;
+  const int lr            = threadIdx.x % lanes_per_row;
+  const int rsub          = threadIdx.x / lanes_per_row;
+  const bool active       = rsub < rows_per_pass;
+  const int fl            = lr * BV;
+  int c_base[BV];
+#pragma unroll
+  for (int v = 0; v < BV; v++) c_base[v] = a.row_pointers[min(f0 + fl + v, f1 - 1)] - bin0;
+  const unsigned long long max_abs = a.qstats[0];
+  const int n_tiles = a.meta->n_tiles;
+  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / a.n_chunks);
+  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / a.n_chunks);
+  int cur_node           = -1;
+  unsigned long long acc = 0;
+  __syncthreads();
+
+  auto flush = [&](int node) {
+    __syncthreads();
+    if (node >= 0) {
+      I64Pair* dst = a.hist.at(node, k, bin0);
+      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+        unsigned long long v = s_hist[i];
+        if (v != 0) {
+          int32_t gv  = static_cast<int32_t>(v >> 32);
+          uint32_t hv = static_cast<uint32_t>(v);
+          if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
+          if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
+          s_hist[i] = 0;
+        }
+      }
+    }
+    __syncthreads();
+  };
+
+  for (int tile = t_begin; tile < t_end; tile++) {
+    int lo = 0, hi = a.n_nodes;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (a.tile_start[mid] <= tile)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
+    const int j       = a.j0 + lo;
+    const int node    = a.level_first + j;
+    const int seg_lo  = a.seg[j];
+    const int seg_hi  = a.seg[j + 1];
+    const int r0      = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
+    const int r1      = min(seg_hi, r0 + kTileRows);
+    const int nrows   = r1 - r0;
+    const bool direct = (seg_hi - seg_lo) < kSmallNodeRows ||
+                        static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
+    if (!direct) {
+      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
+        flush(cur_node);
+        cur_node = node;
+        acc      = 0;
+      }
+      acc += nrows;
+    }
+    if (active) {
+      I64Pair* gdst = a.hist.at(node, k, bin0);
+      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kUnroll) {
+        int row[kUnroll];
+        Word w[kUnroll];
+        int2 q[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          int rr = r + u * rows_per_pass;
+          row[u] = rr < r1 ? a.positions[rr].y : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          if (row[u] >= 0) {
+            const BinT* bp = static_cast<const BinT*>(a.binned) + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
+            w[u]           = *reinterpret_cast<const Word*>(bp);
+            q[u]           = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; u++) {
+          if (row[u] >= 0) {
+            const unsigned long long packed =
+              (static_cast<unsigned long long>(static_cast<uint32_t>(q[u].x)) << 32) |
+              static_cast<unsigned long long>(static_cast<uint32_t>(q[u].y));
+            int rel[BV];
+            unpack_bins<BinT, BV>(w[u], rel);
+#pragma unroll
+            for (int v = 0; v < BV; v++) {
+              if (fl + v < gs) {
+                const int bin = c_base[v] + rel[v];
+                if (direct) {
+                  atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
+                  atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
+                } else {
+                  atomicAdd(&s_hist[bin], packed);
+                }
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+  flush(cur_node);
+}
+
+template <typename KernelT>
+int allow_large_lds(KernelT kernel)
+{
+  LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(kLdsBudget)));
+  return LBT_OK;
+}
+
+// grid: one resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD)
+int grid_for(int n_gk, int64_t n_rows, int n_nodes, int* n_chunks, unsigned* grid)
+{
+  int device = 0, n_cu = 256;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  const int64_t max_tiles = (n_rows + kTileRows - 1) / kTileRows + n_nodes;
+  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / n_gk);
+  per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
+  *n_chunks       = static_cast<int>(per_xcd * 8);
+  *grid           = static_cast<unsigned>(per_xcd * 8 * n_gk);
+  return LBT_OK;
+}
+
+template <typename T, int VEC, typename BinT, bool kWriteBins>
+int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid)
 {
   static bool attr_set = false;
   if (!attr_set) {
-    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(histogram_kernel<T, VEC>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kLdsBudget)));
+    LBT_TRY(allow_large_lds(histogram_kernel<T, VEC, BinT, kWriteBins>));
     attr_set = true;
   }
-  histogram_kernel<T, VEC><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a);
+  histogram_kernel<T, VEC, BinT, kWriteBins><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a);
+  return LBT_OK;
+}
+
+template <typename T, int VEC>
+int launch_search_bins(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid, bool write_bins)
+{
+  if (!write_bins) return launch_search<T, VEC, uint8_t, false>(stream, hs, a, grid);
+  if (hs.bin_bytes == 1) return launch_search<T, VEC, uint8_t, true>(stream, hs, a, grid);
+  return launch_search<T, VEC, uint16_t, true>(stream, hs, a, grid);
+}
+
+template <typename BinT, int BV>
+int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, unsigned grid)
+{
+  static bool attr_set = false;
+  if (!attr_set) {
+    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV>));
+    attr_set = true;
+  }
+  binned_histogram_kernel<BinT, BV><<<grid, kHistThreads, hs.blds_bytes, stream>>>(a);
   return LBT_OK;
 }
 
@@ -431,6 +674,32 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
                                                       b.K, b.hist.node_begin, b.hist.node_end, hs.tile_start,
                                                       hs.meta, b.level_total);
+  }
+  const bool use_cache = hs.binned != nullptr && depth > 0;
+  ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
+  if (use_cache) {
+    BinnedArgs a;
+    a.binned = hs.binned;
+    a.F = b.F;
+    a.qgh = b.qgh;
+    a.K = b.K;
+    a.positions = b.positions;
+    a.seg = b.seg;
+    a.j0 = b.j0;
+    a.n_nodes = b.n_nodes;
+    a.level_first = b.level_first;
+    a.tile_start = hs.tile_start;
+    a.meta = hs.meta;
+    a.row_pointers = b.row_pointers;
+    a.groups = hs.bgroups;
+    a.hist = b.hist;
+    a.qstats = b.qstats;
+    a.n_gk = hs.n_bgroups * b.K;
+    unsigned grid = 0;
+    LBT_TRY(grid_for(a.n_gk, b.n_rows, b.n_nodes, &a.n_chunks, &grid));
+    if (hs.bin_bytes == 1)
+      return hs.bvec == 4 ? launch_binned<uint8_t, 4>(stream, hs, a, grid) : launch_binned<uint8_t, 1>(stream, hs, a, grid);
+    return hs.bvec == 4 ? launch_binned<uint16_t, 4>(stream, hs, a, grid) : launch_binned<uint16_t, 1>(stream, hs, a, grid);
   }
   HistArgs<T> a;
   a.X = static_cast<const T*>(b.X);
@@ -454,24 +723,16 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   a.search_steps = hs.search_steps;
   a.hist = b.hist;
   a.qstats = b.qstats;
+  a.binned = hs.binned;
   a.n_gk = hs.n_groups * b.K;
-
-  int device = 0, n_cu = 256;
-  LBT_HIP(hipGetDevice(&device));
-  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  // one resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD)
-  const int64_t max_tiles = (b.n_rows + kTileRows - 1) / kTileRows + b.n_nodes;
-  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / a.n_gk);
-  per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
-  a.n_chunks      = static_cast<int>(per_xcd * 8);
-  const unsigned grid = static_cast<unsigned>(per_xcd * 8 * a.n_gk);
-
-  ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
+  unsigned grid = 0;
+  LBT_TRY(grid_for(a.n_gk, b.n_rows, b.n_nodes, &a.n_chunks, &grid));
+  const bool write_bins = hs.binned != nullptr && depth == 0;
   if (hs.vec == 4) {
-    if constexpr (sizeof(T) == 4) return launch_kernel<T, 4>(stream, hs, a, grid);
+    if constexpr (sizeof(T) == 4) return launch_search_bins<T, 4>(stream, hs, a, grid, write_bins);
   }
-  if (hs.vec == 2) return launch_kernel<T, 2>(stream, hs, a, grid);
-  return launch_kernel<T, 1>(stream, hs, a, grid);
+  if (hs.vec == 2) return launch_search_bins<T, 2>(stream, hs, a, grid, write_bins);
+  return launch_search_bins<T, 1>(stream, hs, a, grid, write_bins);
 }
 
 }  // namespace
@@ -538,6 +799,45 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const st
     cells >>= 1;
   }
   hs.cells     = cells;
+  if (hs.binned != nullptr) {
+    // groups of the binned kernel: only the packed sub-histogram lives in LDS
+    hs.bin_bytes = max_feature_bins <= 256 ? 1 : 2;
+    hs.bvec      = (F % 4 == 0) ? 4 : 1;
+    std::vector<int32_t> bg;
+    size_t blds = 0;
+    auto packb = [&](int target) {
+      bg.assign(1, 0);
+      blds       = 0;
+      size_t cur = 0;
+      int width  = 0;
+      for (int f = 0; f < F; f += hs.bvec) {
+        size_t cb = 0;
+        for (int i = f; i < std::min(F, f + hs.bvec); i++) cb += static_cast<size_t>(rp[i + 1] - rp[i]) * 8;
+        if (width > 0 && (cur + cb > kLdsBudget || width + hs.bvec > target || (width + hs.bvec) / hs.bvec > max_lanes)) {
+          bg.push_back(f);
+          blds  = std::max(blds, cur);
+          cur   = 0;
+          width = 0;
+        }
+        cur += cb;
+        width += hs.bvec;
+      }
+      bg.push_back(F);
+      blds = std::max(blds, cur);
+    };
+    packb(F + hs.bvec);
+    const int nb_min = static_cast<int>(bg.size()) - 1;
+    int btarget      = (F + nb_min - 1) / nb_min;
+    btarget          = ((btarget + hs.bvec - 1) / hs.bvec) * hs.bvec;
+    packb(btarget);
+    if (blds > kLdsBudget) {
+      hs.binned = nullptr;  // a single feature's histogram cannot exceed the budget, so this does not happen
+    } else {
+      hs.n_bgroups  = static_cast<int>(bg.size()) - 1;
+      hs.blds_bytes = (blds + 15) & ~size_t(15);
+      LBT_HIP(hipMemcpyAsync(hs.bgroups, bg.data(), sizeof(int32_t) * bg.size(), hipMemcpyHostToDevice, stream));
+    }
+  }
   hs.n_groups  = static_cast<int>(groups.size()) - 1;
   hs.lds_bytes = (lds + 15) & ~size_t(15);
   LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));

@@ -266,6 +266,14 @@ struct HistSetup {
   void* cell_invw    = nullptr;  // X dtype [n_features]
   int32_t* tile_start = nullptr;
   LevelMeta* meta    = nullptr;
+  // bin cache: feature-relative bin of every (row, feature), written by the
+  // root-level pass and read by all deeper levels instead of X
+  void* binned         = nullptr;  // uint8 or uint16 [n_rows][n_features], or null (cache off)
+  int bin_bytes        = 0;        // 1 or 2
+  int32_t* bgroups     = nullptr;  // feature groups of the binned kernel [n_bgroups + 1]
+  int n_bgroups        = 0;
+  int bvec             = 1;
+  size_t blds_bytes    = 0;
 };
 
 constexpr int kMaxCells = 2048;
