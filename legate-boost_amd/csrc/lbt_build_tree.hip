@@ -271,13 +271,13 @@ __global__ void __launch_bounds__(kThreads)
   __shared__ int64_t s_g[kThreads / 64];
   __shared__ int64_t s_h[kThreads / 64];
   __shared__ unsigned long long s_m[kThreads / 64];
-  const int k       = blockIdx.y;
-  const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
-  int64_t qg = 0, qh = 0;
+  const int k = blockIdx.y;
+  const double sg = scales[0], sh = scales[1];
+  int64_t sum_g = 0, sum_h = 0;
   unsigned long long mx = 0;
   bool bad = false;
-  if (row < n_rows) {
-    const double sg = scales[0], sh = scales[1];
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t row = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x; row < n_rows; row += stride) {
     double grad = g[row * K + k], hess = h[row * K + k];
     uint32_t x  = minstd_seed(static_cast<uint32_t>(
       static_cast<uint64_t>(gpair_seed(seed, row + row_offset, static_cast<int64_t>(k)))));
@@ -285,38 +285,41 @@ __global__ void __launch_bounds__(kThreads)
     double scaled_hess    = hess * sh;
     double grad_remainder = scaled_grad - floor(scaled_grad);
     double hess_remainder = scaled_hess - floor(scaled_hess);
-    x  = minstd_next(x);
-    qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
-    x  = minstd_next(x);
-    qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
-    bad = qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
+    x = minstd_next(x);
+    int64_t qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
+    x = minstd_next(x);
+    int64_t qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
+    bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
     q_out[row * K + k] = make_int2(static_cast<int>(qg), static_cast<int>(qh));
     unsigned long long ag = static_cast<unsigned long long>(qg < 0 ? -qg : qg);
     unsigned long long ah = static_cast<unsigned long long>(qh < 0 ? -qh : qh);
-    mx = ag > ah ? ag : ah;
+    mx = ag > mx ? ag : mx;
+    mx = ah > mx ? ah : mx;
+    sum_g += qg;
+    sum_h += qh;
   }
   for (int off = 32; off >= 1; off >>= 1) {
-    qg += __shfl_down(qg, off, 64);
-    qh += __shfl_down(qh, off, 64);
+    sum_g += __shfl_down(sum_g, off, 64);
+    sum_h += __shfl_down(sum_h, off, 64);
     unsigned long long o = __shfl_down(mx, off, 64);
     mx = o > mx ? o : mx;
   }
   if (bad) atomicMax(&qstats[1], 1ULL);
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   if (lane == 0) {
-    s_g[wave] = qg;
-    s_h[wave] = qh;
+    s_g[wave] = sum_g;
+    s_h[wave] = sum_h;
     s_m[wave] = mx;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < kThreads / 64; w++) {
-      qg += s_g[w];
-      qh += s_h[w];
+      sum_g += s_g[w];
+      sum_h += s_h[w];
       mx = s_m[w] > mx ? s_m[w] : mx;
     }
-    atomic_add_i64(&node_sums[k].grad, qg);
-    atomic_add_i64(&node_sums[k].hess, qh);
+    atomic_add_i64(&node_sums[k].grad, sum_g);
+    atomic_add_i64(&node_sums[k].hess, sum_h);
     atomicMax(&qstats[0], mx);
   }
 }
@@ -540,7 +543,7 @@ __global__ void proposals_to_double_kernel(const T* p, int n, double* out)
 // by its right rows. Exclusive prefix counts of the "retired" and "left" flags
 // give every destination directly.
 
-constexpr int kPartItems = 4;
+constexpr int kPartItems = 8;
 constexpr int kPartBlock = kThreads * kPartItems;  // rows per workgroup
 
 // pass 1: classify each row (0 retired, 1 left, 2 right) and count per workgroup
@@ -589,38 +592,47 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
-// pass 2: exclusive scan of the per-workgroup counts (single workgroup)
-__global__ void __launch_bounds__(kThreads)
+// pass 2: exclusive scan of the per-workgroup counts (single workgroup of 1024
+// threads; every thread owns a contiguous slice, slices are joined by a wave
+// scan and a scan over the 16 wave totals)
+constexpr int kScanThreads = 1024;
+__global__ void __launch_bounds__(kScanThreads)
   scan_block_counts_kernel(const int2* block_counts, int n_blocks, int2* block_offsets, int2* totals)
 {
-  __shared__ int s_d[kThreads];
-  __shared__ int s_l[kThreads];
-  __shared__ int run_d, run_l;
-  if (threadIdx.x == 0) run_d = run_l = 0;
-  __syncthreads();
-  for (int base = 0; base < n_blocks; base += kThreads) {
-    int b   = base + threadIdx.x;
-    int2 c  = b < n_blocks ? block_counts[b] : make_int2(0, 0);
-    s_d[threadIdx.x] = c.x;
-    s_l[threadIdx.x] = c.y;
-    __syncthreads();
-    for (int off = 1; off < kThreads; off <<= 1) {
-      int vd = threadIdx.x >= off ? s_d[threadIdx.x - off] : 0;
-      int vl = threadIdx.x >= off ? s_l[threadIdx.x - off] : 0;
-      __syncthreads();
-      s_d[threadIdx.x] += vd;
-      s_l[threadIdx.x] += vl;
-      __syncthreads();
-    }
-    if (b < n_blocks) block_offsets[b] = make_int2(run_d + s_d[threadIdx.x] - c.x, run_l + s_l[threadIdx.x] - c.y);
-    __syncthreads();
-    if (threadIdx.x == kThreads - 1) {
-      run_d += s_d[kThreads - 1];
-      run_l += s_l[kThreads - 1];
-    }
-    __syncthreads();
+  __shared__ long long s_wave[kScanThreads / 64];
+  const int per   = (n_blocks + kScanThreads - 1) / kScanThreads;
+  const int begin = threadIdx.x * per;
+  const int end   = min(n_blocks, begin + per);
+  // both counts travel in one 64-bit word: retired in the high half, left in the low half
+  long long mine = 0;
+  for (int b = begin; b < end; b++) {
+    int2 c = block_counts[b];
+    mine += (static_cast<long long>(c.x) << 32) + c.y;
   }
-  if (threadIdx.x == 0) *totals = make_int2(run_d, run_l);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  long long incl = mine;
+  for (int off = 1; off < 64; off <<= 1) {
+    long long o = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    long long run = 0;
+    for (int w = 0; w < kScanThreads / 64; w++) {
+      long long v = s_wave[w];
+      s_wave[w]   = run;
+      run += v;
+    }
+    *totals = make_int2(static_cast<int>(run >> 32), static_cast<int>(run & 0xffffffffLL));
+  }
+  __syncthreads();
+  long long run = s_wave[wave] + incl - mine;
+  for (int b = begin; b < end; b++) {
+    int2 c           = block_counts[b];
+    block_offsets[b] = make_int2(static_cast<int>(run >> 32), static_cast<int>(run & 0xffffffffLL));
+    run += (static_cast<long long>(c.x) << 32) + c.y;
+  }
 }
 
 // Prefix counts (retired, left) in front of index s.
@@ -933,7 +945,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       m = m2;
     }
     scales_kernel<<<1, 64, 0, stream>>>(L.part_a[cur], L.part_b[cur], L.scales, L.qstats);
-    dim3 grid(blocks(N, kThreads), K);
+    dim3 grid(std::min<unsigned>(blocks(N, kThreads), 2048u), K);
     quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(prm.seed),
                                                    L.scales, L.qgh, L.node_sums, L.qstats);
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
@@ -1034,7 +1046,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       const unsigned nb = blocks(N, kPartBlock);
       classify_kernel<T><<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, X, F, feature, split, max_nodes, L.code,
                                                       L.block_counts);
-      scan_block_counts_kernel<<<1, kThreads, 0, stream>>>(L.block_counts, nb, L.block_offsets, L.totals);
+      scan_block_counts_kernel<<<1, kScanThreads, 0, stream>>>(L.block_counts, nb, L.block_offsets, L.totals);
       const int n_parents = static_cast<int>(nodes_in_level);
       child_segments_kernel<<<blocks(static_cast<int64_t>(n_parents) * 64, kThreads), kThreads, 0, stream>>>(
         L.seg[cur_seg], n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[cur_seg ^ 1]);

@@ -105,25 +105,33 @@ struct ProfScope {
 #define LBT_M 2147483647u
 #define LBT_A 48271u
 
+// Reduction modulo the Mersenne prime m = 2^31 - 1 of a value below 2^62:
+// 2^31 == 1 (mod m), so the high part can be folded onto the low part.
+__host__ __device__ inline uint32_t mod_m(uint64_t p)
+{
+  p = (p & LBT_M) + (p >> 31);
+  p = (p & LBT_M) + (p >> 31);
+  return static_cast<uint32_t>(p >= LBT_M ? p - LBT_M : p);
+}
 // thrust::minstd_rand seeding: s mod m, 1 if that is 0.
 __host__ __device__ inline uint32_t minstd_seed(uint32_t s)
 {
-  uint32_t x = s % LBT_M;
+  uint32_t x = mod_m(s);
   return x == 0 ? 1u : x;
 }
 __host__ __device__ inline uint32_t minstd_next(uint32_t x)
 {
-  return static_cast<uint32_t>((static_cast<uint64_t>(x) * LBT_A) % LBT_M);
+  return mod_m(static_cast<uint64_t>(x) * LBT_A);
 }
 __host__ __device__ inline uint32_t minstd_discard(uint32_t x, uint64_t z)
 {
   uint64_t mult = LBT_A, acc = 1;
   while (z > 0) {
-    if (z & 1) acc = (acc * mult) % LBT_M;
-    mult = (mult * mult) % LBT_M;
+    if (z & 1) acc = mod_m(acc * mult);
+    mult = mod_m(mult * mult);
     z >>= 1;
   }
-  return static_cast<uint32_t>((static_cast<uint64_t>(x) * acc) % LBT_M);
+  return mod_m(static_cast<uint64_t>(x) * acc);
 }
 // thrust::uniform_real_distribution<double>(0,1) on one raw draw.
 __host__ __device__ inline double uniform01(uint32_t draw)
