@@ -678,72 +678,76 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
-// pass 4: scatter every pair to its place in the next level's order
+// number of set bits of a 64-bit wave mask below the calling lane
+__device__ inline int prefix_popc(unsigned long long mask)
+{
+  return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0));
+}
+
+// pass 4: scatter every pair to its place in the next level's order. Rows are
+// taken in slabs of one workgroup width (coalesced); inside a slab the ranks
+// come from wave ballots, across waves and slabs from a 32-entry scan.
 __global__ void __launch_bounds__(kThreads)
   scatter_kernel(const int2* pos, int64_t n, const uint8_t* code, const int2* block_offsets,
                  const int32_t* seg, const int2* seg_prefix, const int32_t* seg_next,
                  int level_first, int n_parents, int2* pos_out)
 {
-  __shared__ int s_wave[kThreads / 64];
+  constexpr int kWaves = kThreads / 64;
+  __shared__ int s_cnt[kPartItems * kWaves];  // retired << 16 | left, in row order
   const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // thread t owns the kPartItems consecutive rows base + t*kPartItems ...
+  const int wave = threadIdx.x >> 6;
   int2 p[kPartItems];
   int c[kPartItems];
-  int packed = 0;  // retired count in the high half, left count in the low half
+  int below_d[kPartItems], below_l[kPartItems];
 #pragma unroll
   for (int u = 0; u < kPartItems; u++) {
-    int64_t i = base + static_cast<int64_t>(threadIdx.x) * kPartItems + u;
+    int64_t i = base + u * kThreads + threadIdx.x;
     c[u]      = 3;
     if (i < n) {
       p[u] = pos[i];
       c[u] = code[i];
-      packed += (c[u] == 0 ? (1 << 16) : 0) + (c[u] == 1 ? 1 : 0);
     }
+    unsigned long long md = __ballot(c[u] == 0);
+    unsigned long long ml = __ballot(c[u] == 1);
+    below_d[u]            = prefix_popc(md);
+    below_l[u]            = prefix_popc(ml);
+    if ((threadIdx.x & 63) == 0) s_cnt[u * kWaves + wave] = (__popcll(md) << 16) | __popcll(ml);
   }
-  int incl = packed;
-  for (int off = 1; off < 64; off <<= 1) {
-    int o = __shfl_up(incl, off, 64);
-    if (lane >= off) incl += o;
-  }
-  if (lane == 63) s_wave[wave] = incl;
   __syncthreads();
   if (threadIdx.x == 0) {
     int run = 0;
-    for (int w = 0; w < kThreads / 64; w++) {
-      int v     = s_wave[w];
-      s_wave[w] = run;
+    for (int i = 0; i < kPartItems * kWaves; i++) {
+      int v    = s_cnt[i];
+      s_cnt[i] = run;
       run += v;
     }
   }
   __syncthreads();
-  int excl   = s_wave[wave] + incl - packed;
-  int2 boff  = block_offsets[blockIdx.x];
-  int D      = boff.x + (excl >> 16);
-  int L      = boff.y + (excl & 0xffff);
+  const int2 boff = block_offsets[blockIdx.x];
 #pragma unroll
   for (int u = 0; u < kPartItems; u++) {
-    int64_t i = base + static_cast<int64_t>(threadIdx.x) * kPartItems + u;
+    int64_t i = base + u * kThreads + threadIdx.x;
     if (i < n) {
-      int dest;
-      int new_node;
+      const int excl = s_cnt[u * kWaves + wave];
+      const int D    = boff.x + (excl >> 16) + below_d[u];
+      const int L    = boff.y + (excl & 0xffff) + below_l[u];
+      int dest, new_node;
       if (c[u] == 0) {
         dest     = D;
         new_node = -1;
-        D++;
       } else {
-        int j       = p[u].x - level_first;
-        int s0      = seg[j];
-        int2 sp     = seg_prefix[j];
+        const int j   = p[u].x - level_first;
+        const int s0  = seg[j];
+        const int2 sp = seg_prefix[j];
         if (c[u] == 1) {
           dest     = seg_next[2 * j] + (L - sp.y);
           new_node = left_child(p[u].x);
-          L++;
         } else {
-          int R    = static_cast<int>(i) - D - L;
-          int R0   = s0 - sp.x - sp.y;
-          dest     = seg_next[2 * j + 1] + (R - R0);
-          new_node = right_child(p[u].x);
+          const int R  = static_cast<int>(i) - D - L;
+          const int R0 = s0 - sp.x - sp.y;
+          dest         = seg_next[2 * j + 1] + (R - R0);
+          new_node     = right_child(p[u].x);
         }
       }
       pos_out[dest] = make_int2(new_node, p[u].y);
@@ -778,6 +782,7 @@ struct Layout {
   int32_t* bin_feature;
   int32_t* groups;
   int32_t* bgroups;
+  int32_t* bin_offset;
   void* binned;
   uint16_t* tables;
   void* cell_lo;
@@ -830,8 +835,9 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
   L.groups       = ar.take<int32_t>(F + 1);
   L.bgroups      = ar.take<int32_t>(F + 1);
+  L.bin_offset   = ar.take<int32_t>(F);
   // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
-  L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(N) * F * (S <= 256 ? 1 : 2) + 16)) : nullptr;
+  L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(N) * bin_row_bytes_max(F, S <= 256 ? 1 : 2) + 16)) : nullptr;
   L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
   L.cell_lo      = ar.take<double>(F);
   L.cell_invw    = ar.take<double>(F);
@@ -927,8 +933,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.tile_start = L.tile_start;
   hs.bgroups    = L.bgroups;
   hs.binned     = L.binned;
+  hs.bin_offset = L.bin_offset;
   hs.meta       = L.meta;
-  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, rp, L.proposals, L.row_pointers, X));
+  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, N, rp, L.proposals, L.row_pointers, X));
 
   // ---- quantiser
   {

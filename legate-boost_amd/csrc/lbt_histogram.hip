@@ -13,7 +13,10 @@
 //     HBM once.
 //   * A lane is tied to VEC consecutive features of its group and walks rows, so
 //     the lanes of a wave read consecutive bytes of a row with one 16-byte load
-//     each and keep their features' constants in registers.
+//     each and keep their features' constants in registers. A tile is one pass of
+//     the workgroup (a few rows per lane); the loads of the next tile and the
+//     row indices of the one after are issued before the current tile is
+//     processed, so HBM latency hides behind the bin search.
 //   * Bin search: cell = clamp((x - lo) * invw) indexes the table, which gives the
 //     number of proposals in cells before it; a short forward probe over the
 //     proposals finishes the search. Any monotone cell function is exact here;
@@ -24,6 +27,11 @@
 //     moves to another node. Before the low half or the signed high half could
 //     overflow (rows * max |q| >= 2^31) the sub-histogram is merged early; rows of
 //     tiny nodes go straight to global atomics.
+//   * The root-level pass also stores the feature-relative bin of every value
+//     (one or two bytes). Deeper levels read those instead of X and skip the
+//     search. A cache row holds the groups' slivers one after another, each
+//     padded to a 32-byte sector (128 bytes per row for 100 features in four
+//     groups), so a row gathered at a deep level costs one cache line.
 #include "lbt_internal.h"
 
 #include <algorithm>
@@ -34,16 +42,18 @@ namespace {
 constexpr int kPlanThreads   = 256;
 constexpr int kHistThreads   = 1024;
 constexpr int kSmallNodeRows = 64;  // below this a node goes straight to global atomics
-constexpr int kUnroll        = 4;
+constexpr int kUnroll        = 4;   // rows per lane and tile, search kernel
+constexpr int kBinnedUnroll  = 8;   // rows per lane and tile, binned kernel
 constexpr int kLinearProbes  = 4;   // forward probes before falling back to a binary search
 constexpr size_t kLdsBudget  = 160 * 1024 - 512;
 
 // For the nodes [j0, j1) of the current level (level-local indices): decides
-// which are built (build_tree.h:92-104) and cuts their row segments into tiles.
-// tile_start[j - j0] = first tile of node j; tile_start[j1 - j0] = total.
+// which are built (build_tree.h:92-104) and cuts their row segments into tiles
+// of tile_rows rows. tile_start[j - j0] = first tile of node j;
+// tile_start[j1 - j0] = total.
 __global__ void __launch_bounds__(kPlanThreads)
   plan_tiles_kernel(int j0, int j1, int level_first, const int32_t* seg, const I64Pair* node_sums,
-                    int K, int hist_node_begin, int hist_node_end, int32_t* tile_start,
+                    int K, int hist_node_begin, int hist_node_end, int tile_rows, int32_t* tile_start,
                     LevelMeta* meta, LevelMeta* level_total)
 {
   __shared__ int s_scan[kPlanThreads];
@@ -65,7 +75,7 @@ __global__ void __launch_bounds__(kPlanThreads)
       int parent = parent_of(node);
       bool pex   = parent >= hist_node_begin && parent < hist_node_end;
       built      = compute_histogram_bin(node, node_sums, K, pex);
-      tiles      = built ? (rows + kTileRows - 1) / kTileRows : 0;
+      tiles      = built ? (rows + tile_rows - 1) / tile_rows : 0;
     }
     s_scan[threadIdx.x] = tiles;
     __syncthreads();
@@ -164,12 +174,8 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-template <typename T>
-struct HistArgs {
-  const T* X;
-  int F;
-  const int2* qgh;  // [N][K] packed int32 (grad, hess)
-  int K;
+// What both kernels need to walk the tiles of a batch.
+struct TileWalk {
   const int2* positions;  // (node,row) sorted by node
   const int32_t* seg;     // level-local segment starts
   int j0;                 // first level-local node of the batch
@@ -177,6 +183,61 @@ struct HistArgs {
   int level_first;        // global index of level-local node 0
   const int32_t* tile_start;
   const LevelMeta* meta;
+  int tile_rows;
+  int rpp;       // rows per pass of a workgroup (tile_rows / rows per lane)
+  int n_gk;      // groups * outputs
+  int n_chunks;  // row-tile ranges
+  const unsigned long long* qstats;
+};
+
+struct Tile {
+  int node;
+  int r0, r1;
+  int seg_rows;
+};
+
+// Node and row range of a tile. `hint` is the batch-local node of the previous
+// lookup (tiles are visited in order, so the node index only moves forward); a
+// negative hint starts with a binary search. All values are uniform over the
+// workgroup.
+__device__ inline Tile tile_lookup(const TileWalk& w, int tile, int& hint)
+{
+  int lo;
+  if (hint < 0) {
+    // last j with tile_start[j] <= tile
+    lo     = 0;
+    int hi = w.n_nodes;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (w.tile_start[mid] <= tile)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
+  } else {
+    lo = hint;
+    while (w.tile_start[lo + 1] <= tile) lo++;
+  }
+  hint             = lo;
+  const int j      = w.j0 + lo;
+  const int seg_lo = w.seg[j];
+  const int seg_hi = w.seg[j + 1];
+  Tile t;
+  t.node     = w.level_first + j;
+  t.r0       = seg_lo + (tile - w.tile_start[lo]) * w.tile_rows;
+  t.r1       = min(seg_hi, t.r0 + w.tile_rows);
+  t.seg_rows = seg_hi - seg_lo;
+  return t;
+}
+
+template <typename T>
+struct HistArgs {
+  TileWalk w;
+  const T* X;
+  int F;
+  int64_t n_rows;
+  const int2* qgh;  // [N][K] packed int32 (grad, hess)
+  int K;
   const T* proposals;
   const int32_t* row_pointers;
   const int32_t* groups;  // feature groups: [n_groups+1]
@@ -185,11 +246,10 @@ struct HistArgs {
   const T* cell_invw;
   int cells;
   int search_steps;
-  int n_gk;      // groups * outputs
-  int n_chunks;  // row-tile ranges
   HistView hist;
-  const unsigned long long* qstats;
-  void* binned;  // bin cache (written by the root pass, read by the binned kernel)
+  void* binned;               // bin cache, written when kWriteBins
+  const int32_t* bin_offset;  // [F] element offset of a feature inside a cache row
+  int bin_pitch;              // elements per cache row
 };
 
 template <typename T, int VEC>
@@ -229,19 +289,36 @@ __device__ inline int count_less(const T* p, int n, T x, int steps)
   return lo;
 }
 
+
+// Merge of the packed LDS sub-histogram into the int64 histogram of a node.
+__device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst)
+{
+  for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+    unsigned long long v = s_hist[i];
+    if (v != 0) {
+      int32_t gv  = static_cast<int32_t>(v >> 32);
+      uint32_t hv = static_cast<uint32_t>(v);
+      if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
+      if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
+      s_hist[i] = 0;
+    }
+  }
+}
+
 template <typename T, int VEC, typename BinT, bool kWriteBins>
 __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
 {
   using Vec = typename VecOf<T, VEC>::type;
   extern __shared__ unsigned char smem_raw[];
+  const TileWalk& w = a.w;
 
   // workgroup -> (row-tile range, group, output). Linear workgroup ids are dealt
   // round-robin to the 8 XCDs, so id % 8 is the XCD; within an XCD consecutive
   // slots enumerate (group, output) of one row-tile range.
   const int xcd   = blockIdx.x & 7;
   const int slot  = blockIdx.x >> 3;
-  const int gk    = slot % a.n_gk;
-  const int chunk = (slot / a.n_gk) * 8 + xcd;
+  const int gk    = slot % w.n_gk;
+  const int chunk = (slot / w.n_gk) * 8 + xcd;
   const int group = gk / a.K;
   const int k     = gk % a.K;
 
@@ -268,10 +345,9 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
   }
 
   const int lanes_per_row = (gs + VEC - 1) / VEC;
-  const int rows_per_pass = kHistThreads / lanes_per_row;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
-  const bool active       = rsub < rows_per_pass;
+  const bool active       = rsub < w.rpp;
   const int fl            = lr * VEC;  // first group-local feature of this lane
 
   T c_lo[VEC], c_invw[VEC];
@@ -286,144 +362,155 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
     c_end[v]  = a.row_pointers[f + 1] - bin0;
   }
   const T cmax = static_cast<T>(C - 1);
-  const unsigned long long max_abs = a.qstats[0];
+  const unsigned long long max_abs = w.qstats[0];
+  // unused elements between this group's sliver and the next one in a cache row
+  const int pad = kWriteBins ? (f1 < a.F ? a.bin_offset[f1] : a.bin_pitch) - (a.bin_offset[f0] + gs) : 0;
+  // this lane's place in a row of the bin cache
+  BinT* const bin_base = kWriteBins ? static_cast<BinT*>(a.binned) + a.bin_offset[min(f0 + fl, f1 - 1)] : nullptr;
 
-  const int n_tiles = a.meta->n_tiles;
-  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / a.n_chunks);
-  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / a.n_chunks);
+  const int n_tiles = w.meta->n_tiles;
+  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
+  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / w.n_chunks);
 
   int cur_node           = -1;
   unsigned long long acc = 0;  // rows added to the LDS copy since it was last merged
   __syncthreads();
 
-  auto flush = [&](int node) {
-    __syncthreads();
-    if (node >= 0) {
-      I64Pair* dst = a.hist.at(node, k, bin0);
-      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
-        unsigned long long v = s_hist[i];
-        if (v != 0) {
-          int32_t gv  = static_cast<int32_t>(v >> 32);
-          uint32_t hv = static_cast<uint32_t>(v);
-          if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
-          if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
-          s_hist[i] = 0;
-        }
+  auto load_rows = [&](const Tile& t, int (&row)[kUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      int rr = t.r0 + rsub + u * w.rpp;
+      row[u] = (active && rr < t.r1) ? w.positions[rr].y : -1;
+    }
+  };
+  auto load_data = [&](const int (&row)[kUnroll], Vec (&xv)[kUnroll], int2 (&q)[kUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      if (row[u] >= 0) {
+        const T* xp = a.X + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
+        if constexpr (VEC == 1)
+          xv[u] = *xp;
+        else
+          xv[u] = *reinterpret_cast<const Vec*>(xp);
+        q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
       }
     }
-    __syncthreads();
   };
 
+  Tile tc{}, tn{}, tnn{};
+  int hint = -1;
+  int row_c[kUnroll], row_n[kUnroll], row_nn[kUnroll];
+  Vec x_c[kUnroll], x_n[kUnroll];
+  int2 q_c[kUnroll], q_n[kUnroll];
+#pragma unroll
+  for (int u = 0; u < kUnroll; u++) row_c[u] = row_n[u] = row_nn[u] = -1;
+  if (t_begin < t_end) {
+    tc = tile_lookup(w, t_begin, hint);
+    load_rows(tc, row_c);
+    load_data(row_c, x_c, q_c);
+  }
+  if (t_begin + 1 < t_end) {
+    tn = tile_lookup(w, t_begin + 1, hint);
+    load_rows(tn, row_n);
+  }
+
   for (int tile = t_begin; tile < t_end; tile++) {
-    // node of this tile: last j with tile_start[j] <= tile (uniform over the workgroup)
-    int lo = 0, hi = a.n_nodes;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (a.tile_start[mid] <= tile)
-        lo = mid;
-      else
-        hi = mid - 1;
+    // issue the loads of the next tile and the row indices of the one after
+    if (tile + 1 < t_end) load_data(row_n, x_n, q_n);
+    if (tile + 2 < t_end) {
+      tnn = tile_lookup(w, tile + 2, hint);
+      load_rows(tnn, row_nn);
     }
-    const int j       = a.j0 + lo;
-    const int node    = a.level_first + j;
-    const int seg_lo  = a.seg[j];
-    const int seg_hi  = a.seg[j + 1];
-    const int r0      = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
-    const int r1      = min(seg_hi, r0 + kTileRows);
-    const int nrows   = r1 - r0;
-    const bool direct = (seg_hi - seg_lo) < kSmallNodeRows ||
+
+    const int nrows   = tc.r1 - tc.r0;
+    const bool direct = tc.seg_rows < kSmallNodeRows ||
                         static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
     if (!direct) {
-      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
-        flush(cur_node);
-        cur_node = node;
+      if (tc.node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
+        __syncthreads();
+        if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
+        __syncthreads();
+        cur_node = tc.node;
         acc      = 0;
       }
       acc += nrows;
     }
-    if (active) {
-      I64Pair* gdst = a.hist.at(node, k, bin0);
-      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kUnroll) {
-        int row[kUnroll];
-        Vec xv[kUnroll];
-        int2 q[kUnroll];
+    I64Pair* gdst = a.hist.at(tc.node, k, bin0);
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          int rr = r + u * rows_per_pass;
-          row[u] = rr < r1 ? a.positions[rr].y : -1;
+    for (int u = 0; u < kUnroll; u++) {
+      if (row_c[u] >= 0) {
+        const unsigned long long packed =
+          (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
+          static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+        T xs[VEC];
+        if constexpr (VEC == 1) {
+          xs[0] = x_c[u];
+        } else if constexpr (VEC == 2) {
+          xs[0] = x_c[u].x;
+          xs[1] = x_c[u].y;
+        } else {
+          xs[0] = x_c[u].x;
+          xs[1] = x_c[u].y;
+          xs[2] = x_c[u].z;
+          xs[3] = x_c[u].w;
         }
+        BinT rel[VEC];
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          if (row[u] >= 0) {
-            const T* xp = a.X + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
-            if constexpr (VEC == 1)
-              xv[u] = *xp;
-            else
-              xv[u] = *reinterpret_cast<const Vec*>(xp);
-            q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
+        for (int v = 0; v < VEC; v++) {
+          const T x = xs[v];
+          int bin   = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+          bool lt   = s_prop[bin] < x;
+          int probes = 0;
+          while (__any(lt)) {
+            bin += lt ? 1 : 0;
+            if (++probes == kLinearProbes) {
+              // crowded cell: finish with a binary search over the rest of the feature
+              bin += count_less(s_prop + bin, c_end[v] - bin, x, a.search_steps);
+              break;
+            }
+            lt = s_prop[bin] < x;
+          }
+          rel[v] = static_cast<BinT>(bin - c_prop[v]);
+          if (direct) {
+            atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
+            atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
+          } else {
+            atomicAdd(&s_hist[bin], packed);
           }
         }
-#pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          if (row[u] >= 0) {
-            const unsigned long long packed =
-              (static_cast<unsigned long long>(static_cast<uint32_t>(q[u].x)) << 32) |
-              static_cast<unsigned long long>(static_cast<uint32_t>(q[u].y));
-            T xs[VEC];
-            if constexpr (VEC == 1) {
-              xs[0] = xv[u];
-            } else if constexpr (VEC == 2) {
-              xs[0] = xv[u].x;
-              xs[1] = xv[u].y;
+        if constexpr (kWriteBins) {
+          if (k == 0 && f0 + fl < f1) {
+            BinT* bp = bin_base + static_cast<int64_t>(row_c[u]) * a.bin_pitch;
+            if constexpr (VEC == 4 && sizeof(BinT) == 1) {
+              *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
+                                                 (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
             } else {
-              xs[0] = xv[u].x;
-              xs[1] = xv[u].y;
-              xs[2] = xv[u].z;
-              xs[3] = xv[u].w;
-            }
-            BinT rel[VEC];
 #pragma unroll
-            for (int v = 0; v < VEC; v++) {
-              const T x = xs[v];
-              int bin   = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
-              bool lt   = s_prop[bin] < x;
-              int probes = 0;
-              while (__any(lt)) {
-                bin += lt ? 1 : 0;
-                if (++probes == kLinearProbes) {
-                  // crowded cell: finish with a binary search over the rest of the feature
-                  bin += count_less(s_prop + bin, c_end[v] - bin, x, a.search_steps);
-                  break;
-                }
-                lt = s_prop[bin] < x;
-              }
-              rel[v] = static_cast<BinT>(bin - c_prop[v]);
-              if (direct) {
-                atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
-                atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
-              } else {
-                atomicAdd(&s_hist[bin], packed);
-              }
+              for (int v = 0; v < VEC; v++)
+                if (f0 + fl + v < f1) bp[v] = rel[v];
             }
-            if constexpr (kWriteBins) {
-              if (k == 0 && f0 + fl < f1) {
-                BinT* bp = static_cast<BinT*>(a.binned) + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
-                if constexpr (VEC == 4 && sizeof(BinT) == 1) {
-                  *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
-                                                     (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
-                } else {
-#pragma unroll
-                  for (int v = 0; v < VEC; v++)
-                    if (f0 + fl + v < f1) bp[v] = rel[v];
-                }
-              }
+            // the lane that holds the group's last features also clears the padding up to
+            // the next sliver, so that whole sectors are written
+            if (fl + VEC >= gs) {
+              for (int i = gs - fl; i < gs - fl + pad; i++) bp[i] = 0;
             }
           }
         }
       }
     }
+    // rotate the pipeline
+    tc = tn;
+    tn = tnn;
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      row_c[u] = row_n[u];
+      row_n[u] = row_nn[u];
+      x_c[u]   = x_n[u];
+      q_c[u]   = q_n[u];
+    }
   }
-  flush(cur_node);
+  __syncthreads();
+  if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
 }
 
 // Deeper levels: the bins of every (row, feature) are already known, so a lane
@@ -467,23 +554,15 @@ __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int
 }
 
 struct BinnedArgs {
+  TileWalk w;
   const void* binned;
-  int F;
+  const int32_t* bin_offset;  // [F] element offset of a feature inside a cache row
+  int bin_pitch;              // elements per cache row
   const int2* qgh;
   int K;
-  const int2* positions;
-  const int32_t* seg;
-  int j0;
-  int n_nodes;
-  int level_first;
-  const int32_t* tile_start;
-  const LevelMeta* meta;
   const int32_t* row_pointers;
   const int32_t* groups;
-  int n_gk;
-  int n_chunks;
   HistView hist;
-  const unsigned long long* qstats;
 };
 
 template <typename BinT, int BV>
@@ -491,10 +570,11 @@ __global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedAr
 {
   using Word = typename BinVec<BinT, BV>::type;
   extern __shared__ unsigned char smem_raw[];
+  const TileWalk& w = a.w;
   const int xcd   = blockIdx.x & 7;
   const int slot  = blockIdx.x >> 3;
-  const int gk    = slot % a.n_gk;
-  const int chunk = (slot / a.n_gk) * 8 + xcd;
+  const int gk    = slot % w.n_gk;
+  const int chunk = (slot / w.n_gk) * 8 + xcd;
   const int group = gk / a.K;
   const int k     = gk % a.K;
   const int f0 = a.groups[group], f1 = a.groups[group + 1];
@@ -505,111 +585,112 @@ __global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedAr
   for (int i = threadIdx.x; i < nb; i += kHistThreads) s_hist[i] = 0;
 
   const int lanes_per_row = (gs + BV - 1) / BV;
-  const int rows_per_pass = kHistThreads / lanes_per_row;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
-  const bool active       = rsub < rows_per_pass;
+  const bool active       = rsub < w.rpp;
   const int fl            = lr * BV;
+  const int f_lane        = min(f0 + fl, f1 - 1);
+  const BinT* const my_bins = static_cast<const BinT*>(a.binned) + a.bin_offset[f_lane];
+  const int my_stride       = a.bin_pitch;
   int c_base[BV];
 #pragma unroll
   for (int v = 0; v < BV; v++) c_base[v] = a.row_pointers[min(f0 + fl + v, f1 - 1)] - bin0;
-  const unsigned long long max_abs = a.qstats[0];
-  const int n_tiles = a.meta->n_tiles;
-  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / a.n_chunks);
-  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / a.n_chunks);
+  const unsigned long long max_abs = w.qstats[0];
+  const int n_tiles = w.meta->n_tiles;
+  const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
+  const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / w.n_chunks);
   int cur_node           = -1;
   unsigned long long acc = 0;
   __syncthreads();
 
-  auto flush = [&](int node) {
-    __syncthreads();
-    if (node >= 0) {
-      I64Pair* dst = a.hist.at(node, k, bin0);
-      for (int i = threadIdx.x; i < nb; i += kHistThreads) {
-        unsigned long long v = s_hist[i];
-        if (v != 0) {
-          int32_t gv  = static_cast<int32_t>(v >> 32);
-          uint32_t hv = static_cast<uint32_t>(v);
-          if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
-          if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
-          s_hist[i] = 0;
-        }
+  auto load_rows = [&](const Tile& t, int (&row)[kBinnedUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kBinnedUnroll; u++) {
+      int rr = t.r0 + rsub + u * w.rpp;
+      row[u] = (active && rr < t.r1) ? w.positions[rr].y : -1;
+    }
+  };
+  auto load_data = [&](const int (&row)[kBinnedUnroll], Word (&bw)[kBinnedUnroll], int2 (&q)[kBinnedUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kBinnedUnroll; u++) {
+      if (row[u] >= 0) {
+        bw[u] = *reinterpret_cast<const Word*>(my_bins + static_cast<int64_t>(row[u]) * my_stride);
+        q[u]  = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
       }
     }
-    __syncthreads();
   };
 
+  Tile tc{}, tn{}, tnn{};
+  int hint = -1;
+  int row_c[kBinnedUnroll], row_n[kBinnedUnroll], row_nn[kBinnedUnroll];
+  Word b_c[kBinnedUnroll], b_n[kBinnedUnroll];
+  int2 q_c[kBinnedUnroll], q_n[kBinnedUnroll];
+#pragma unroll
+  for (int u = 0; u < kBinnedUnroll; u++) row_c[u] = row_n[u] = row_nn[u] = -1;
+  if (t_begin < t_end) {
+    tc = tile_lookup(w, t_begin, hint);
+    load_rows(tc, row_c);
+    load_data(row_c, b_c, q_c);
+  }
+  if (t_begin + 1 < t_end) {
+    tn = tile_lookup(w, t_begin + 1, hint);
+    load_rows(tn, row_n);
+  }
+
   for (int tile = t_begin; tile < t_end; tile++) {
-    int lo = 0, hi = a.n_nodes;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (a.tile_start[mid] <= tile)
-        lo = mid;
-      else
-        hi = mid - 1;
+    if (tile + 1 < t_end) load_data(row_n, b_n, q_n);
+    if (tile + 2 < t_end) {
+      tnn = tile_lookup(w, tile + 2, hint);
+      load_rows(tnn, row_nn);
     }
-    const int j       = a.j0 + lo;
-    const int node    = a.level_first + j;
-    const int seg_lo  = a.seg[j];
-    const int seg_hi  = a.seg[j + 1];
-    const int r0      = seg_lo + (tile - a.tile_start[lo]) * kTileRows;
-    const int r1      = min(seg_hi, r0 + kTileRows);
-    const int nrows   = r1 - r0;
-    const bool direct = (seg_hi - seg_lo) < kSmallNodeRows ||
+    const int nrows   = tc.r1 - tc.r0;
+    const bool direct = tc.seg_rows < kSmallNodeRows ||
                         static_cast<unsigned long long>(nrows) * max_abs > 2147483647ULL;
     if (!direct) {
-      if (node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
-        flush(cur_node);
-        cur_node = node;
+      if (tc.node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
+        __syncthreads();
+        if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
+        __syncthreads();
+        cur_node = tc.node;
         acc      = 0;
       }
       acc += nrows;
     }
-    if (active) {
-      I64Pair* gdst = a.hist.at(node, k, bin0);
-      for (int r = r0 + rsub; r < r1; r += rows_per_pass * kUnroll) {
-        int row[kUnroll];
-        Word w[kUnroll];
-        int2 q[kUnroll];
+    I64Pair* gdst = a.hist.at(tc.node, k, bin0);
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          int rr = r + u * rows_per_pass;
-          row[u] = rr < r1 ? a.positions[rr].y : -1;
-        }
+    for (int u = 0; u < kBinnedUnroll; u++) {
+      if (row_c[u] >= 0) {
+        const unsigned long long packed =
+          (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
+          static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+        int rel[BV];
+        unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          if (row[u] >= 0) {
-            const BinT* bp = static_cast<const BinT*>(a.binned) + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
-            w[u]           = *reinterpret_cast<const Word*>(bp);
-            q[u]           = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; u++) {
-          if (row[u] >= 0) {
-            const unsigned long long packed =
-              (static_cast<unsigned long long>(static_cast<uint32_t>(q[u].x)) << 32) |
-              static_cast<unsigned long long>(static_cast<uint32_t>(q[u].y));
-            int rel[BV];
-            unpack_bins<BinT, BV>(w[u], rel);
-#pragma unroll
-            for (int v = 0; v < BV; v++) {
-              if (fl + v < gs) {
-                const int bin = c_base[v] + rel[v];
-                if (direct) {
-                  atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q[u].x));
-                  atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q[u].y));
-                } else {
-                  atomicAdd(&s_hist[bin], packed);
-                }
-              }
+        for (int v = 0; v < BV; v++) {
+          if (fl + v < gs) {
+            const int bin = c_base[v] + rel[v];
+            if (direct) {
+              atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
+              atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
+            } else {
+              atomicAdd(&s_hist[bin], packed);
             }
           }
         }
       }
     }
+    tc = tn;
+    tn = tnn;
+#pragma unroll
+    for (int u = 0; u < kBinnedUnroll; u++) {
+      row_c[u] = row_n[u];
+      row_n[u] = row_nn[u];
+      b_c[u]   = b_n[u];
+      q_c[u]   = q_n[u];
+    }
   }
-  flush(cur_node);
+  __syncthreads();
+  if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
 }
 
 template <typename KernelT>
@@ -617,20 +698,6 @@ int allow_large_lds(KernelT kernel)
 {
   LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(kLdsBudget)));
-  return LBT_OK;
-}
-
-// grid: one resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD)
-int grid_for(int n_gk, int64_t n_rows, int n_nodes, int* n_chunks, unsigned* grid)
-{
-  int device = 0, n_cu = 256;
-  LBT_HIP(hipGetDevice(&device));
-  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  const int64_t max_tiles = (n_rows + kTileRows - 1) / kTileRows + n_nodes;
-  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / n_gk);
-  per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
-  *n_chunks       = static_cast<int>(per_xcd * 8);
-  *grid           = static_cast<unsigned>(per_xcd * 8 * n_gk);
   return LBT_OK;
 }
 
@@ -666,67 +733,80 @@ int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, 
   return LBT_OK;
 }
 
+// One resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD).
+int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_groups, int rpp, int unroll, unsigned* grid)
+{
+  int device = 0, n_cu = 256;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  w.positions   = b.positions;
+  w.seg         = b.seg;
+  w.j0          = b.j0;
+  w.n_nodes     = b.n_nodes;
+  w.level_first = b.level_first;
+  w.tile_start  = hs.tile_start;
+  w.meta        = hs.meta;
+  w.rpp         = rpp;
+  w.tile_rows   = rpp * unroll;
+  w.n_gk        = n_groups * b.K;
+  w.qstats      = b.qstats;
+  const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
+  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / w.n_gk);
+  per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
+  w.n_chunks      = static_cast<int>(per_xcd * 8);
+  *grid           = static_cast<unsigned>(per_xcd * 8 * w.n_gk);
+  return LBT_OK;
+}
+
 template <typename T>
 int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth)
 {
+  const bool use_cache = hs.binned != nullptr && depth > 0;
+  TileWalk w;
+  unsigned grid = 0;
+  LBT_TRY(fill_walk(w, hs, b, use_cache ? hs.n_bgroups : hs.n_groups, use_cache ? hs.brpp : hs.rpp,
+                    use_cache ? kBinnedUnroll : kUnroll, &grid));
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
     plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
-                                                      b.K, b.hist.node_begin, b.hist.node_end, hs.tile_start,
-                                                      hs.meta, b.level_total);
+                                                      b.K, b.hist.node_begin, b.hist.node_end, w.tile_rows,
+                                                      hs.tile_start, hs.meta, b.level_total);
   }
-  const bool use_cache = hs.binned != nullptr && depth > 0;
   ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   if (use_cache) {
     BinnedArgs a;
-    a.binned = hs.binned;
-    a.F = b.F;
-    a.qgh = b.qgh;
-    a.K = b.K;
-    a.positions = b.positions;
-    a.seg = b.seg;
-    a.j0 = b.j0;
-    a.n_nodes = b.n_nodes;
-    a.level_first = b.level_first;
-    a.tile_start = hs.tile_start;
-    a.meta = hs.meta;
+    a.w            = w;
+    a.binned       = hs.binned;
+    a.bin_offset   = hs.bin_offset;
+    a.bin_pitch    = hs.bin_pitch;
+    a.qgh          = b.qgh;
+    a.K            = b.K;
     a.row_pointers = b.row_pointers;
-    a.groups = hs.bgroups;
-    a.hist = b.hist;
-    a.qstats = b.qstats;
-    a.n_gk = hs.n_bgroups * b.K;
-    unsigned grid = 0;
-    LBT_TRY(grid_for(a.n_gk, b.n_rows, b.n_nodes, &a.n_chunks, &grid));
+    a.groups       = hs.bgroups;
+    a.hist         = b.hist;
     if (hs.bin_bytes == 1)
       return hs.bvec == 4 ? launch_binned<uint8_t, 4>(stream, hs, a, grid) : launch_binned<uint8_t, 1>(stream, hs, a, grid);
     return hs.bvec == 4 ? launch_binned<uint16_t, 4>(stream, hs, a, grid) : launch_binned<uint16_t, 1>(stream, hs, a, grid);
   }
   HistArgs<T> a;
-  a.X = static_cast<const T*>(b.X);
-  a.F = b.F;
-  a.qgh = b.qgh;
-  a.K = b.K;
-  a.positions = b.positions;
-  a.seg = b.seg;
-  a.j0 = b.j0;
-  a.n_nodes = b.n_nodes;
-  a.level_first = b.level_first;
-  a.tile_start = hs.tile_start;
-  a.meta = hs.meta;
-  a.proposals = static_cast<const T*>(b.proposals);
+  a.w            = w;
+  a.X            = static_cast<const T*>(b.X);
+  a.F            = b.F;
+  a.n_rows       = b.n_rows;
+  a.qgh          = b.qgh;
+  a.K            = b.K;
+  a.proposals    = static_cast<const T*>(b.proposals);
   a.row_pointers = b.row_pointers;
-  a.groups = hs.groups;
-  a.tables = hs.tables;
-  a.cell_lo = static_cast<const T*>(hs.cell_lo);
-  a.cell_invw = static_cast<const T*>(hs.cell_invw);
-  a.cells = hs.cells;
+  a.groups       = hs.groups;
+  a.tables       = hs.tables;
+  a.cell_lo      = static_cast<const T*>(hs.cell_lo);
+  a.cell_invw    = static_cast<const T*>(hs.cell_invw);
+  a.cells        = hs.cells;
   a.search_steps = hs.search_steps;
-  a.hist = b.hist;
-  a.qstats = b.qstats;
-  a.binned = hs.binned;
-  a.n_gk = hs.n_groups * b.K;
-  unsigned grid = 0;
-  LBT_TRY(grid_for(a.n_gk, b.n_rows, b.n_nodes, &a.n_chunks, &grid));
+  a.hist         = b.hist;
+  a.binned       = hs.binned;
+  a.bin_offset   = hs.bin_offset;
+  a.bin_pitch    = hs.bin_pitch;
   const bool write_bins = hs.binned != nullptr && depth == 0;
   if (hs.vec == 4) {
     if constexpr (sizeof(T) == 4) return launch_search_bins<T, 4>(stream, hs, a, grid, write_bins);
@@ -735,18 +815,68 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   return launch_search_bins<T, 1>(stream, hs, a, grid, write_bins);
 }
 
+// Packs consecutive features, `unit` at a time, into groups whose LDS need
+// (bytes_of(feature)) stays within the budget; a second pass balances widths.
+template <typename BytesOf>
+size_t pack_groups(int F, int unit, BytesOf bytes_of, std::vector<int32_t>& groups)
+{
+  const int max_lanes = kHistThreads / 2;  // at least two rows per pass
+  size_t lds          = 0;
+  auto pack = [&](int target) {
+    groups.assign(1, 0);
+    lds        = 0;
+    size_t cur = 0;
+    int width  = 0;
+    for (int f = 0; f < F; f += unit) {
+      size_t cb = 0;
+      for (int i = f; i < std::min(F, f + unit); i++) cb += bytes_of(i);
+      if (width > 0 && (cur + cb > kLdsBudget || width + unit > target || (width + unit) / unit > max_lanes)) {
+        groups.push_back(f);
+        lds   = std::max(lds, cur);
+        cur   = 0;
+        width = 0;
+      }
+      cur += cb;
+      width += unit;
+    }
+    groups.push_back(F);
+    lds = std::max(lds, cur);
+  };
+  pack(F + unit);  // fewest groups the LDS allows
+  const int n_min = static_cast<int>(groups.size()) - 1;
+  int target      = (F + n_min - 1) / n_min;
+  target          = ((target + unit - 1) / unit) * unit;
+  pack(target);    // same count, balanced widths
+  return lds;
+}
+
+int rows_per_pass(const std::vector<int32_t>& groups, int vec)
+{
+  int rpp = kHistThreads;
+  for (size_t g = 0; g + 1 < groups.size(); g++) {
+    int lanes = (groups[g + 1] - groups[g] + vec - 1) / vec;
+    rpp       = std::min(rpp, kHistThreads / lanes);
+  }
+  return rpp;
+}
+
 }  // namespace
 
-int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const std::vector<int32_t>& rp,
-                 const void* proposals, const int32_t* row_pointers, const void* X)
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t n_rows,
+                 const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
+                 const void* X)
 {
+  (void)n_rows;
   const size_t elem = is_f64 ? 8 : 4;
   hs.is_f64         = is_f64;
   hs.n_features     = F;
   // widest aligned vector of features a lane can load
   int vec = is_f64 ? 2 : 4;
   while (vec > 1 && (F % vec != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0)) vec >>= 1;
-  hs.vec = vec;
+  hs.vec  = vec;
+  hs.bvec = (F % 4 == 0) ? 4 : 1;
+  // group boundaries suit both the search kernel and the cached-bin layout
+  const int unit = hs.binned != nullptr ? std::max(vec, hs.bvec) : vec;
   int max_feature_bins = 1;
   for (int f = 0; f < F; f++) max_feature_bins = std::max(max_feature_bins, rp[f + 1] - rp[f]);
   hs.search_steps = 0;
@@ -757,40 +887,10 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const st
   while (cells < 4 * max_feature_bins && cells < kMaxCells) cells <<= 1;
   std::vector<int32_t> groups;
   size_t lds = 0;
-  const int max_lanes = kHistThreads / 2;  // at least two rows per pass
   for (;;) {
-    // bytes of LDS a feature needs: proposals + packed sub-histogram + its table
-    auto chunk_bytes = [&](int f) {
-      size_t bytes = 0;
-      for (int i = f; i < std::min(F, f + vec); i++)
-        bytes += static_cast<size_t>(rp[i + 1] - rp[i]) * (8 + elem) + static_cast<size_t>(cells) * 2;
-      return bytes;
-    };
-    // features are packed in units of `vec`; `target` caps the width of a group
-    auto pack = [&](int target) {
-      groups.assign(1, 0);
-      lds        = 0;
-      size_t cur = 0;
-      int width  = 0;
-      for (int f = 0; f < F; f += vec) {
-        size_t cb = chunk_bytes(f);
-        if (width > 0 && (cur + cb > kLdsBudget || width + vec > target || (width + vec) / vec > max_lanes)) {
-          groups.push_back(f);
-          lds   = std::max(lds, cur);
-          cur   = 0;
-          width = 0;
-        }
-        cur += cb;
-        width += vec;
-      }
-      groups.push_back(F);
-      lds = std::max(lds, cur);
-    };
-    pack(F + vec);  // fewest groups the LDS allows
-    const int n_min = static_cast<int>(groups.size()) - 1;
-    int target      = (F + n_min - 1) / n_min;
-    target          = ((target + vec - 1) / vec) * vec;
-    pack(target);   // same count, balanced widths
+    lds = pack_groups(F, unit, [&](int f) {
+      return static_cast<size_t>(rp[f + 1] - rp[f]) * (8 + elem) + static_cast<size_t>(cells) * 2;
+    }, groups);
     if (lds <= kLdsBudget) break;
     if (cells <= 64) {
       set_error("a feature group does not fit the LDS (%zu bytes)", lds);
@@ -799,48 +899,47 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const st
     cells >>= 1;
   }
   hs.cells     = cells;
-  if (hs.binned != nullptr) {
-    // groups of the binned kernel: only the packed sub-histogram lives in LDS
-    hs.bin_bytes = max_feature_bins <= 256 ? 1 : 2;
-    hs.bvec      = (F % 4 == 0) ? 4 : 1;
-    std::vector<int32_t> bg;
-    size_t blds = 0;
-    auto packb = [&](int target) {
-      bg.assign(1, 0);
-      blds       = 0;
-      size_t cur = 0;
-      int width  = 0;
-      for (int f = 0; f < F; f += hs.bvec) {
-        size_t cb = 0;
-        for (int i = f; i < std::min(F, f + hs.bvec); i++) cb += static_cast<size_t>(rp[i + 1] - rp[i]) * 8;
-        if (width > 0 && (cur + cb > kLdsBudget || width + hs.bvec > target || (width + hs.bvec) / hs.bvec > max_lanes)) {
-          bg.push_back(f);
-          blds  = std::max(blds, cur);
-          cur   = 0;
-          width = 0;
-        }
-        cur += cb;
-        width += hs.bvec;
-      }
-      bg.push_back(F);
-      blds = std::max(blds, cur);
-    };
-    packb(F + hs.bvec);
-    const int nb_min = static_cast<int>(bg.size()) - 1;
-    int btarget      = (F + nb_min - 1) / nb_min;
-    btarget          = ((btarget + hs.bvec - 1) / hs.bvec) * hs.bvec;
-    packb(btarget);
-    if (blds > kLdsBudget) {
-      hs.binned = nullptr;  // a single feature's histogram cannot exceed the budget, so this does not happen
-    } else {
-      hs.n_bgroups  = static_cast<int>(bg.size()) - 1;
-      hs.blds_bytes = (blds + 15) & ~size_t(15);
-      LBT_HIP(hipMemcpyAsync(hs.bgroups, bg.data(), sizeof(int32_t) * bg.size(), hipMemcpyHostToDevice, stream));
-    }
-  }
   hs.n_groups  = static_cast<int>(groups.size()) - 1;
   hs.lds_bytes = (lds + 15) & ~size_t(15);
+  hs.rpp       = rows_per_pass(groups, vec);
   LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
+  if (hs.binned != nullptr) {
+    hs.bin_bytes = max_feature_bins <= 256 ? 1 : 2;
+    // groups of the binned kernel: only the packed sub-histogram lives in LDS
+    std::vector<int32_t> bg;
+    size_t blds = pack_groups(F, hs.bvec, [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; }, bg);
+    if (blds > kLdsBudget) {
+      set_error("a feature's histogram does not fit the LDS (%zu bytes)", blds);
+      return LBT_ERR_UNSUPPORTED;
+    }
+    hs.n_bgroups  = static_cast<int>(bg.size()) - 1;
+    hs.blds_bytes = (blds + 15) & ~size_t(15);
+    hs.brpp       = rows_per_pass(bg, hs.bvec);
+    LBT_HIP(hipMemcpyAsync(hs.bgroups, bg.data(), sizeof(int32_t) * bg.size(), hipMemcpyHostToDevice, stream));
+    // a cache row: the search groups' slivers one after another, each padded to `align`
+    // bytes (a 32-byte sector if the row budget allows, else less)
+    std::vector<int32_t> off(F);
+    for (int align = 32;; align >>= 1) {
+      int64_t at = 0;
+      for (size_t g = 0; g + 1 < groups.size(); g++) {
+        for (int f = groups[g]; f < groups[g + 1]; f++) off[f] = static_cast<int32_t>(at + (f - groups[g]));
+        int64_t bytes = static_cast<int64_t>(groups[g + 1] - groups[g]) * hs.bin_bytes;
+        bytes         = (bytes + align - 1) / align * align;
+        at += bytes / hs.bin_bytes;
+      }
+      if (at * hs.bin_bytes <= bin_row_bytes_max(F, hs.bin_bytes) || align <= 4) {
+        hs.bin_pitch = static_cast<int>(at);
+        break;
+      }
+    }
+    if (static_cast<int64_t>(hs.bin_pitch) * hs.bin_bytes > bin_row_bytes_max(F, hs.bin_bytes)) {
+      set_error("bin cache row of %d bytes exceeds the workspace share", hs.bin_pitch * hs.bin_bytes);
+      return LBT_ERR_WORKSPACE;
+    }
+    LBT_HIP(hipMemcpyAsync(hs.bin_offset, off.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
+    // the host vectors must outlive the asynchronous copies
+    LBT_HIP(hipStreamSynchronize(stream));
+  }
   ProfScope ps(LBT_PROF_PROPOSALS, stream);
   if (is_f64)
     build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,

@@ -254,7 +254,6 @@ struct LevelMeta {
   long long built_nodes;
 };
 
-constexpr int kTileRows = 1024;  // rows of one node between two bookkeeping steps
 
 // Per-tree state of the histogram stage: feature groups sized for the LDS of
 // one workgroup and, per feature, a table that maps a value to the first
@@ -282,9 +281,21 @@ struct HistSetup {
   int n_bgroups        = 0;
   int bvec             = 1;
   size_t blds_bytes    = 0;
+  int32_t* bin_offset  = nullptr;  // [n_features] element offset of a feature inside a cache row
+  int bin_pitch        = 0;        // elements per cache row
+  int rpp              = 0;        // rows per workgroup pass, search kernel
+  int brpp             = 0;        // rows per workgroup pass, binned kernel
 };
 
 constexpr int kMaxCells = 2048;
+
+// Upper bound on the bytes of one row of the bin cache (features plus sector padding
+// between groups); the workspace reserves n_rows times this.
+inline int64_t bin_row_bytes_max(int n_features, int bin_bytes)
+{
+  int64_t raw = static_cast<int64_t>(n_features) * bin_bytes;
+  return (raw + raw / 4 + 31) / 32 * 32 + 64;
+}
 
 struct HistBatch {
   const void* X;
@@ -307,8 +318,9 @@ struct HistBatch {
 
 // Chooses groups / table size from the host copy of the row pointers and builds
 // the tables on the device.
-int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, const std::vector<int32_t>& rp,
-                 const void* proposals, const int32_t* row_pointers, const void* X);
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t n_rows,
+                 const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
+                 const void* X);
 // Plans tiles for the batch and launches the histogram kernel.
 int hist_launch(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth);
 
