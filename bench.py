@@ -32,6 +32,8 @@ def parse():
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--rows", type=int, default=0, help="override the number of rows (0 = the configuration's)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reference-flow", action="store_true",
+                    help="update the training predictions with a PredictTask per round (as the reference loop does) instead of the row->leaf map that BuildTreeTask can return")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     return ap.parse_args()
 
@@ -129,8 +131,13 @@ def bench_training(args):
             g = (pred - yc) * lr
             h = torch.ones_like(pred)
         seed = int(rs.randint(0, 2**31))
-        r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
-        pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
+        if args.reference_flow:
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
+            pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
+        else:
+            # same values as PredictTask on the training rows (checked bit for bit in the tests)
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True)
+            pred.add_(r.leaf_value[r.row_leaf.long()])
         return r
 
     def loss():
@@ -180,6 +187,7 @@ def bench_training(args):
                            n, f, k),
             "rows": n, "features": f, "outputs": k, "max_depth": depth, "split_samples": S,
             "loss_before": loss0, "loss_after": loss1,
+            "prediction_update": "PredictTask" if args.reference_flow else "row->leaf map from BuildTreeTask",
         },
         "roofline": {
             "bound": "hbm",

@@ -66,6 +66,8 @@ typedef struct lbt_build_taps {
   int64_t* node_sums;           /* [max_nodes*n_outputs*2] */
   int32_t* positions;           /* [n_rows*2] (node,row) after the last update */
   int32_t* positions_per_level; /* [max_depth*n_rows*2]; slot d = order used at depth d */
+  int32_t* row_leaf;            /* [n_rows] node each local row ends in; leaf[row_leaf[r]] is what
+                                   PredictTask returns for training row r */
   int64_t* histogram;           /* [nodes][n_outputs][n_bins][2] of the last histogram buffer */
   int64_t histogram_capacity;   /* in: int64 elements available at `histogram` */
   /* host outputs */

@@ -487,7 +487,8 @@ __global__ void __launch_bounds__(64)
   split_apply_kernel(HistView hist, I64Pair* node_sums, const int32_t* bin_feature,
                      const double* proposals_as_double, const double* scales, double l1, double l2,
                      int node_begin, int n_chunks, const Cand* partial, double* leaf,
-                     int32_t* feature, double* split, double* gain_out)
+                     int32_t* feature, double* split, double* gain_out, const int32_t* row_pointers,
+                     int32_t* split_bin)
 {
   __shared__ Cand s_c[1];
   __shared__ Cand s_best;
@@ -517,9 +518,11 @@ __global__ void __launch_bounds__(64)
     leaf[static_cast<int64_t>(rc) * K + k] = calculate_leaf_value(
       static_cast<double>(rs.grad) * inv_g, static_cast<double>(rs.hess) * inv_h, l1, l2);
     if (k == 0) {
-      feature[node]  = bin_feature[best.bin];
-      split[node]    = proposals_as_double[best.bin];
-      gain_out[node] = best.gain;
+      const int ft    = bin_feature[best.bin];
+      feature[node]   = ft;
+      split[node]     = proposals_as_double[best.bin];
+      gain_out[node]  = best.gain;
+      split_bin[node] = best.bin - row_pointers[ft];
     }
   }
 }
@@ -590,6 +593,120 @@ __global__ void __launch_bounds__(kThreads)
     }
     block_counts[blockIdx.x] = make_int2(nd, nl);
   }
+}
+
+// Feature-major copy of the bin cache: out[f][row]. One workgroup turns 128
+// cache rows x up to 64 features through LDS so that both sides move whole
+// 4-byte words. `offset`/`pitch` describe a cache row in elements.
+constexpr int kTransRows = 128;
+constexpr int kTransFeat = kTransposeFeatures;
+template <typename BinT>
+__global__ void __launch_bounds__(kThreads)
+  transpose_bins_kernel(const BinT* cache, const int32_t* offset, int pitch, int64_t n_rows, int F,
+                        int64_t out_stride, BinT* out)
+{
+  extern __shared__ unsigned char smem_raw[];
+  uint32_t* s_words   = reinterpret_cast<uint32_t*>(smem_raw);
+  const int64_t r0    = blockIdx.x * static_cast<int64_t>(kTransRows);
+  const int fa        = blockIdx.y * kTransFeat;
+  const int fb        = min(F, fa + kTransFeat);
+  constexpr int per_w = 4 / sizeof(BinT);  // elements per 32-bit word
+  const int e0        = offset[fa] / per_w * per_w;  // first element staged, word aligned
+  const int e1        = offset[fb - 1] + 1;
+  const int n_words   = (e1 - e0 + per_w - 1) / per_w;
+  const int lpitch    = n_words + 1;  // odd pitch spreads a column over the LDS banks
+  for (int i = threadIdx.x; i < kTransRows * n_words; i += kThreads) {
+    int r = i / n_words, wi = i % n_words;
+    uint32_t v = 0;
+    if (r0 + r < n_rows)
+      v = reinterpret_cast<const uint32_t*>(cache + (r0 + r) * pitch + e0)[wi];
+    s_words[r * lpitch + wi] = v;
+  }
+  __syncthreads();
+  const BinT* s_el       = reinterpret_cast<const BinT*>(s_words);
+  constexpr int row_sets = kTransRows / per_w;  // output words per feature
+  for (int i = threadIdx.x; i < (fb - fa) * row_sets; i += kThreads) {
+    int f = fa + i / row_sets, rs = i % row_sets;
+    int col = offset[f] - e0;
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < per_w; j++) {
+      uint32_t b = s_el[static_cast<size_t>(rs * per_w + j) * lpitch * per_w + col];
+      word |= b << (8 * sizeof(BinT) * j);
+    }
+    reinterpret_cast<uint32_t*>(out + f * out_stride + r0)[rs] = word;
+  }
+}
+
+// pass 1 when the feature-major bins exist: x <= proposals[b] holds exactly when the
+// row's bin (first proposal that is not below x) is <= b, so the split feature's bin
+// decides the side and consecutive rows of a node read consecutive bytes.
+template <typename BinT>
+__global__ void __launch_bounds__(kThreads)
+  classify_bins_kernel(const int2* pos, int64_t n, const BinT* bins_t, int64_t bins_stride,
+                       const int32_t* feature, const int32_t* split_bin, int max_nodes, uint8_t* code,
+                       int2* block_counts)
+{
+  __shared__ int s_d[kThreads / 64];
+  __shared__ int s_l[kThreads / 64];
+  const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  int nd = 0, nl = 0;
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    int64_t i = base + u * kThreads + threadIdx.x;
+    if (i < n) {
+      int2 p = pos[i];
+      int c  = 0;
+      if (p.x >= 0 && p.x < max_nodes) {
+        int ft = feature[p.x];
+        if (ft != -1) c = static_cast<int>(bins_t[ft * bins_stride + p.y]) <= split_bin[p.x] ? 1 : 2;
+      }
+      code[i] = static_cast<uint8_t>(c);
+      nd += c == 0;
+      nl += c == 1;
+    }
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    nd += __shfl_down(nd, off, 64);
+    nl += __shfl_down(nl, off, 64);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_d[threadIdx.x >> 6] = nd;
+    s_l[threadIdx.x >> 6] = nl;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / 64; w++) {
+      nd += s_d[w];
+      nl += s_l[w];
+    }
+    block_counts[blockIdx.x] = make_int2(nd, nl);
+  }
+}
+
+// Leaf of every row that is still in a node after the last level: the node itself if it
+// did not split, else the child the row falls into.
+template <typename T, typename BinT>
+__global__ void __launch_bounds__(kThreads)
+  final_leaf_kernel(const int2* pos, int64_t n, const T* X, int F, const BinT* bins_t, int64_t bins_stride,
+                    const int32_t* feature, const double* split, const int32_t* split_bin, int max_nodes,
+                    int32_t* row_leaf)
+{
+  int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (i >= n) return;
+  int2 p = pos[i];
+  if (p.x < 0 || p.x >= max_nodes) return;  // retired earlier: recorded when it retired
+  int node = p.x;
+  int ft   = feature[node];
+  if (ft != -1) {
+    bool left;
+    if (bins_t != nullptr)
+      left = static_cast<int>(bins_t[ft * bins_stride + p.y]) <= split_bin[node];
+    else
+      left = static_cast<double>(X[static_cast<int64_t>(p.y) * F + ft]) <= split[node];
+    node = left ? left_child(node) : right_child(node);
+  }
+  row_leaf[p.y] = node;
 }
 
 // pass 2: exclusive scan of the per-workgroup counts (single workgroup of 1024
@@ -691,7 +808,7 @@ __device__ inline int prefix_popc(unsigned long long mask)
 __global__ void __launch_bounds__(kThreads)
   scatter_kernel(const int2* pos, int64_t n, const uint8_t* code, const int2* block_offsets,
                  const int32_t* seg, const int2* seg_prefix, const int32_t* seg_next,
-                 int level_first, int n_parents, int2* pos_out)
+                 int level_first, int n_parents, int2* pos_out, int32_t* row_leaf)
 {
   constexpr int kWaves = kThreads / 64;
   __shared__ int s_cnt[kPartItems * kWaves];  // retired << 16 | left, in row order
@@ -736,6 +853,8 @@ __global__ void __launch_bounds__(kThreads)
       if (c[u] == 0) {
         dest     = D;
         new_node = -1;
+        // a row that retires now sits in a leaf: remember which
+        if (row_leaf != nullptr && p[u].x >= 0) row_leaf[p[u].y] = p[u].x;
       } else {
         const int j   = p[u].x - level_first;
         const int s0  = seg[j];
@@ -795,6 +914,9 @@ struct Layout {
   int2* pos[2];
   int32_t* seg[2];
   uint8_t* code;
+  int32_t* split_bin;
+  void* bins_t;
+  int64_t bins_t_stride;
   int2* block_counts;
   int2* block_offsets;
   int2* totals;
@@ -853,6 +975,11 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.seg[0] = ar.take<int32_t>(level_nodes + 1);
   L.seg[1] = ar.take<int32_t>(level_nodes + 1);
   L.code   = ar.take<uint8_t>(N);
+  L.split_bin = ar.take<int32_t>(max_nodes);
+  // feature-major bins for the position update (needs the bin cache)
+  L.bins_t_stride = (N + kTransRows - 1) / kTransRows * kTransRows;
+  L.bins_t = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(F) * L.bins_t_stride * (S <= 256 ? 1 : 2)))
+                            : nullptr;
   const int64_t n_pblocks = (N + kPartBlock - 1) / kPartBlock;
   L.block_counts  = ar.take<int2>(n_pblocks);
   L.block_offsets = ar.take<int2>(n_pblocks);
@@ -1000,6 +1127,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   }
 
   int cur_pos = 0, cur_seg = 0;
+  // the feature-major bins serve the position updates of levels 0 .. max_depth-2
+  const bool use_bins_t = hs.binned != nullptr && L.bins_t != nullptr;
+  int32_t* row_leaf     = taps ? taps->row_leaf : nullptr;
   const int n_chunks = (B + kSplitChunk - 1) / kSplitChunk;
   for (int depth = 0; depth < max_depth; depth++) {
     if (taps && taps->positions_per_level)
@@ -1045,26 +1175,66 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
                                                          prm.min_split_gain, batch_begin, n_chunks, L.partial);
         split_apply_kernel<<<n_nodes, 64, 0, stream>>>(hv, L.node_sums, L.bin_feature, L.proposals_d, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization, batch_begin,
-                                                       n_chunks, L.partial, leaf, feature, split, gain);
+                                                       n_chunks, L.partial, leaf, feature, split, gain, L.row_pointers,
+                                                       L.split_bin);
       }
+    }
+    if (depth == 0 && use_bins_t) {
+      // feature-major copy of the bins the root pass has just cached
+      ProfScope ps(LBT_PROF_POSITIONS, stream);
+      dim3 grid(blocks(N, kTransRows), blocks(F, kTransFeat));
+      const size_t lds_t = static_cast<size_t>(kTransRows) * ((hs.trans_span * hs.bin_bytes + 3) / 4 + 2) * 4;
+      if (lds_t > 64 * 1024) {
+        set_error("bin transpose needs %zu bytes of LDS", lds_t);
+        return LBT_ERR_UNSUPPORTED;
+      }
+      if (hs.bin_bytes == 1)
+        transpose_bins_kernel<uint8_t><<<grid, kThreads, lds_t, stream>>>(
+          static_cast<const uint8_t*>(hs.binned), hs.bin_offset, hs.bin_pitch, N, F, L.bins_t_stride,
+          static_cast<uint8_t*>(L.bins_t));
+      else
+        transpose_bins_kernel<uint16_t><<<grid, kThreads, lds_t, stream>>>(
+          static_cast<const uint16_t*>(hs.binned), hs.bin_offset, hs.bin_pitch, N, F, L.bins_t_stride,
+          static_cast<uint16_t*>(L.bins_t));
     }
     if (depth < max_depth - 1) {
       ProfScope ps(LBT_PROF_POSITIONS, stream, static_cast<double>(N) * (8 + 8 + 2 + 64));
       const unsigned nb = blocks(N, kPartBlock);
-      classify_kernel<T><<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, X, F, feature, split, max_nodes, L.code,
-                                                      L.block_counts);
+      if (use_bins_t && hs.bin_bytes == 1)
+        classify_bins_kernel<uint8_t><<<nb, kThreads, 0, stream>>>(
+          L.pos[cur_pos], N, static_cast<const uint8_t*>(L.bins_t), L.bins_t_stride, feature, L.split_bin,
+          max_nodes, L.code, L.block_counts);
+      else if (use_bins_t)
+        classify_bins_kernel<uint16_t><<<nb, kThreads, 0, stream>>>(
+          L.pos[cur_pos], N, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, L.split_bin,
+          max_nodes, L.code, L.block_counts);
+      else
+        classify_kernel<T><<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, X, F, feature, split, max_nodes, L.code,
+                                                        L.block_counts);
       scan_block_counts_kernel<<<1, kScanThreads, 0, stream>>>(L.block_counts, nb, L.block_offsets, L.totals);
       const int n_parents = static_cast<int>(nodes_in_level);
       child_segments_kernel<<<blocks(static_cast<int64_t>(n_parents) * 64, kThreads), kThreads, 0, stream>>>(
         L.seg[cur_seg], n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[cur_seg ^ 1]);
       scatter_kernel<<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, L.code, L.block_offsets, L.seg[cur_seg],
                                                   L.seg_prefix, L.seg[cur_seg ^ 1], level_first, n_parents,
-                                                  L.pos[cur_pos ^ 1]);
+                                                  L.pos[cur_pos ^ 1], row_leaf);
       cur_pos ^= 1;
       cur_seg ^= 1;
     }
   }
 
+  if (row_leaf != nullptr) {
+    ProfScope ps(LBT_PROF_POSITIONS, stream);
+    const bool bt = use_bins_t && max_depth >= 2;
+    if (bt && hs.bin_bytes == 2)
+      final_leaf_kernel<T, uint16_t><<<blocks(N, kThreads), kThreads, 0, stream>>>(
+        L.pos[cur_pos], N, X, F, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, split,
+        L.split_bin, max_nodes, row_leaf);
+    else
+      final_leaf_kernel<T, uint8_t><<<blocks(N, kThreads), kThreads, 0, stream>>>(
+        L.pos[cur_pos], N, X, F, bt ? static_cast<const uint8_t*>(L.bins_t) : nullptr, L.bins_t_stride, feature,
+        split, L.split_bin, max_nodes, row_leaf);
+  }
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
     write_hessian_kernel<<<blocks(static_cast<int64_t>(max_nodes) * K, kThreads), kThreads, 0, stream>>>(

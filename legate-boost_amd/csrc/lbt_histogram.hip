@@ -936,6 +936,11 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t 
       set_error("bin cache row of %d bytes exceeds the workspace share", hs.bin_pitch * hs.bin_bytes);
       return LBT_ERR_WORKSPACE;
     }
+    hs.trans_span = 0;
+    for (int fa = 0; fa < F; fa += kTransposeFeatures) {
+      int fb = std::min(F, fa + kTransposeFeatures);
+      hs.trans_span = std::max(hs.trans_span, off[fb - 1] + 1 - off[fa] / 4 * 4);
+    }
     LBT_HIP(hipMemcpyAsync(hs.bin_offset, off.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
     // the host vectors must outlive the asynchronous copies
     LBT_HIP(hipStreamSynchronize(stream));

@@ -283,11 +283,13 @@ struct HistSetup {
   size_t blds_bytes    = 0;
   int32_t* bin_offset  = nullptr;  // [n_features] element offset of a feature inside a cache row
   int bin_pitch        = 0;        // elements per cache row
+  int trans_span       = 0;        // widest stretch of a cache row that kTransposeFeatures features cover
   int rpp              = 0;        // rows per workgroup pass, search kernel
   int brpp             = 0;        // rows per workgroup pass, binned kernel
 };
 
 constexpr int kMaxCells = 2048;
+constexpr int kTransposeFeatures = 64;  // features one workgroup of the bin transpose handles
 
 // Upper bound on the bytes of one row of the bin cache (features plus sector padding
 // between groups); the workspace reserves n_rows times this.

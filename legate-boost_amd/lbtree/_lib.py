@@ -38,6 +38,7 @@ class BuildTaps(C.Structure):
         ("node_sums", C.c_void_p),
         ("positions", C.c_void_p),
         ("positions_per_level", C.c_void_p),
+        ("row_leaf", C.c_void_p),
         ("histogram", C.c_void_p),
         ("histogram_capacity", C.c_int64),
         ("n_bins", C.c_int32),

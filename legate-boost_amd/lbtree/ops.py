@@ -56,7 +56,7 @@ class BuildResult:
 
 def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0, l2_regularization=1.0,
                min_split_gain=0.0, feature_set=None, dataset_rows=None, row_offset=0, hist_cache_bytes=0,
-               taps=False, taps_levels=False):
+               taps=False, taps_levels=False, row_leaf=False):
     """BUILD_TREE (legateboost/models/tree.py:104-191). Returns a BuildResult with the five task
     outputs as CUDA tensors; with taps=True also the observation points."""
     X = _check_x(X)
@@ -90,8 +90,13 @@ def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0
             raise _lib.LbtError("feature_set must have shape (n_features,)")
     tp = None
     keep = []
-    if taps:
+    if taps or row_leaf:
         tp = _lib.BuildTaps()
+    if row_leaf:
+        # leaf of every training row, so that the caller can update its predictions without a traversal
+        r.row_leaf = torch.empty(n, dtype=torch.int32, device=dev)
+        tp.row_leaf = r.row_leaf.data_ptr()
+    if taps:
         r.proposals_buf = torch.empty(f * split_samples, dtype=X.dtype, device=dev)
         r.row_pointers = torch.empty(f + 1, dtype=torch.int32, device=dev)
         r.quantised = torch.empty((n, k, 2), dtype=torch.int32, device=dev)

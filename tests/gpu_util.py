@@ -55,11 +55,21 @@ def assert_tree_parity(gr, cr, *, levels=False, leaf_exact=True):
     assert np.array_equal(gr.level_built_nodes, cr.level_built_nodes)
 
 
+def check_row_leaf(gr, X):
+    """leaf_value[row_leaf] must be exactly what PredictTask returns for the training rows."""
+    from lbtree import ops
+
+    want = ops.predict(X, [(gr.leaf_value, gr.feature, gr.split_value)], gr.leaf_value.shape[1])
+    got = gr.leaf_value[gr.row_leaf.long()]
+    assert torch.equal(got, want)
+
+
 def both(X, g, h, *, levels=False, **kw):
     cr = orc.build_tree(X, g, h, max_depth=kw["max_depth"], split_samples=kw["split_samples"], seed=kw["seed"],
                         l1=kw.get("l1_regularization", 0.0), l2=kw.get("l2_regularization", 1.0),
                         min_split_gain=kw.get("min_split_gain", 0.0), feature_set=kw.get("feature_set"),
                         hist_cache_bytes=kw.get("hist_cache_bytes", 0), want_levels=levels)
-    gr = gpu_build(X, g, h, taps_levels=levels, **kw)
+    gr = gpu_build(X, g, h, taps_levels=levels, row_leaf=True, **kw)
     torch.cuda.synchronize()
+    check_row_leaf(gr, X)
     return gr, cr
