@@ -203,6 +203,9 @@ def bench_training(args):
             "levels": levels,
         },
         "kernel_ms_per_round": {c: prof[c]["ms"] / args.steps for c in _lib.PROF_CLASSES},
+        "binning": {"ms": prof["binning"]["ms"] / args.steps, "GB": prof["binning"]["bytes"] / args.steps / 1e9,
+                    "GBps": (prof["binning"]["bytes"] / (prof["binning"]["ms"] * 1e-3) / 1e9)
+                    if prof["binning"]["ms"] > 0 else 0.0},
     }
     if not args.no_cpu_baseline:
         ns = min(n, 500_000 if cfg != 1 else n)

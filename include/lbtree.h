@@ -146,7 +146,8 @@ int lbt_update_tree(void* stream, const void* X, int32_t x_dtype, int64_t n_rows
 #define LBT_PROF_POSITIONS 5
 #define LBT_PROF_OTHER 6
 #define LBT_PROF_PREDICT 7
-#define LBT_PROF_CLASSES 8
+#define LBT_PROF_BINNING 8 /* root pass that caches the bin of every feature value */
+#define LBT_PROF_CLASSES 9
 
 typedef struct lbt_profile {
   /* per kernel class: launches timed, summed GPU time (ms, HIP events on the

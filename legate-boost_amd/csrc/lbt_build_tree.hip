@@ -596,45 +596,45 @@ __global__ void __launch_bounds__(kThreads)
 }
 
 // Feature-major copy of the bin cache: out[f][row]. One workgroup turns 128
-// cache rows x up to 64 features through LDS so that both sides move whole
-// 4-byte words. `offset`/`pitch` describe a cache row in elements.
+// rows of one group through LDS, 64 features at a time, so that both sides move
+// whole 4-byte words. `base`/`stride` locate a feature's bins in the cache.
 constexpr int kTransRows = 128;
 constexpr int kTransFeat = kTransposeFeatures;
 template <typename BinT>
 __global__ void __launch_bounds__(kThreads)
-  transpose_bins_kernel(const BinT* cache, const int32_t* offset, int pitch, int64_t n_rows, int F,
-                        int64_t out_stride, BinT* out)
+  transpose_bins_kernel(const BinT* cache, const int32_t* groups, const int64_t* base, const int32_t* stride,
+                        int64_t n_rows, int64_t out_stride, BinT* out)
 {
-  extern __shared__ unsigned char smem_raw[];
-  uint32_t* s_words   = reinterpret_cast<uint32_t*>(smem_raw);
-  const int64_t r0    = blockIdx.x * static_cast<int64_t>(kTransRows);
-  const int fa        = blockIdx.y * kTransFeat;
-  const int fb        = min(F, fa + kTransFeat);
-  constexpr int per_w = 4 / sizeof(BinT);  // elements per 32-bit word
-  const int e0        = offset[fa] / per_w * per_w;  // first element staged, word aligned
-  const int e1        = offset[fb - 1] + 1;
-  const int n_words   = (e1 - e0 + per_w - 1) / per_w;
-  const int lpitch    = n_words + 1;  // odd pitch spreads a column over the LDS banks
-  for (int i = threadIdx.x; i < kTransRows * n_words; i += kThreads) {
-    int r = i / n_words, wi = i % n_words;
-    uint32_t v = 0;
-    if (r0 + r < n_rows)
-      v = reinterpret_cast<const uint32_t*>(cache + (r0 + r) * pitch + e0)[wi];
-    s_words[r * lpitch + wi] = v;
-  }
-  __syncthreads();
-  const BinT* s_el       = reinterpret_cast<const BinT*>(s_words);
-  constexpr int row_sets = kTransRows / per_w;  // output words per feature
-  for (int i = threadIdx.x; i < (fb - fa) * row_sets; i += kThreads) {
-    int f = fa + i / row_sets, rs = i % row_sets;
-    int col = offset[f] - e0;
-    uint32_t word = 0;
-#pragma unroll
-    for (int j = 0; j < per_w; j++) {
-      uint32_t b = s_el[static_cast<size_t>(rs * per_w + j) * lpitch * per_w + col];
-      word |= b << (8 * sizeof(BinT) * j);
+  constexpr int per_w  = 4 / sizeof(BinT);                  // elements per 32-bit word
+  constexpr int lpitch = kTransFeat / per_w + 1;            // odd word pitch spreads a column over the banks
+  __shared__ uint32_t s_words[kTransRows * lpitch];
+  const int64_t r0 = blockIdx.x * static_cast<int64_t>(kTransRows);
+  const int f0 = groups[blockIdx.y], f1 = groups[blockIdx.y + 1];
+  const int pitch = stride[f0];
+  for (int fa = f0; fa < f1; fa += kTransFeat) {
+    const int fb      = min(f1, fa + kTransFeat);
+    const int n_words = (fb - fa + per_w - 1) / per_w;
+    const BinT* src   = cache + base[fa];  // 4-byte aligned: group starts and fa - f0 are multiples of 4 bytes
+    __syncthreads();
+    for (int i = threadIdx.x; i < kTransRows * n_words; i += kThreads) {
+      int r = i / n_words, wi = i % n_words;
+      uint32_t v = 0;
+      if (r0 + r < n_rows) v = reinterpret_cast<const uint32_t*>(src + (r0 + r) * pitch)[wi];
+      s_words[r * lpitch + wi] = v;
     }
-    reinterpret_cast<uint32_t*>(out + f * out_stride + r0)[rs] = word;
+    __syncthreads();
+    const BinT* s_el       = reinterpret_cast<const BinT*>(s_words);
+    constexpr int row_sets = kTransRows / per_w;  // output words per feature
+    for (int i = threadIdx.x; i < (fb - fa) * row_sets; i += kThreads) {
+      int f = fa + i / row_sets, rs = i % row_sets;
+      uint32_t word = 0;
+#pragma unroll
+      for (int j = 0; j < per_w; j++) {
+        uint32_t b = s_el[static_cast<size_t>(rs * per_w + j) * lpitch * per_w + (f - fa)];
+        word |= b << (8 * sizeof(BinT) * j);
+      }
+      reinterpret_cast<uint32_t*>(out + f * out_stride + r0)[rs] = word;
+    }
   }
 }
 
@@ -900,8 +900,8 @@ struct Layout {
   int32_t* row_pointers;
   int32_t* bin_feature;
   int32_t* groups;
-  int32_t* bgroups;
-  int32_t* bin_offset;
+  int64_t* bin_base;
+  int32_t* bin_stride;
   void* binned;
   uint16_t* tables;
   void* cell_lo;
@@ -923,6 +923,7 @@ struct Layout {
   int2* seg_prefix;
   // histogram
   int32_t* tile_start;
+  int4* tiles;
   LevelMeta* meta;
   LevelMeta* level_totals;
   Cand* partial;
@@ -956,8 +957,8 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.row_pointers = ar.take<int32_t>(F + 1);
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
   L.groups       = ar.take<int32_t>(F + 1);
-  L.bgroups      = ar.take<int32_t>(F + 1);
-  L.bin_offset   = ar.take<int32_t>(F);
+  L.bin_base     = ar.take<int64_t>(F);
+  L.bin_stride   = ar.take<int32_t>(F);
   // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
   L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(N) * bin_row_bytes_max(F, S <= 256 ? 1 : 2) + 16)) : nullptr;
   L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
@@ -986,6 +987,8 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.totals        = ar.take<int2>(1);
   L.seg_prefix    = ar.take<int2>(level_nodes);
   L.tile_start    = ar.take<int32_t>(level_nodes + 1);
+  // a tile holds at least 8 rows (two rows per pass, four passes); every node adds at most one partial tile
+  L.tiles         = ar.take<int4>(N / 8 + level_nodes + 1);
   L.meta          = ar.take<LevelMeta>(1);
   L.level_totals  = ar.take<LevelMeta>(max_depth > 0 ? max_depth : 1);
   const int64_t max_chunks = (static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk;
@@ -1058,9 +1061,10 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.cell_lo    = L.cell_lo;
   hs.cell_invw  = L.cell_invw;
   hs.tile_start = L.tile_start;
-  hs.bgroups    = L.bgroups;
+  hs.tiles      = L.tiles;
   hs.binned     = L.binned;
-  hs.bin_offset = L.bin_offset;
+  hs.bin_base   = L.bin_base;
+  hs.bin_stride = L.bin_stride;
   hs.meta       = L.meta;
   LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, N, rp, L.proposals, L.row_pointers, X));
 
@@ -1182,19 +1186,14 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     if (depth == 0 && use_bins_t) {
       // feature-major copy of the bins the root pass has just cached
       ProfScope ps(LBT_PROF_POSITIONS, stream);
-      dim3 grid(blocks(N, kTransRows), blocks(F, kTransFeat));
-      const size_t lds_t = static_cast<size_t>(kTransRows) * ((hs.trans_span * hs.bin_bytes + 3) / 4 + 2) * 4;
-      if (lds_t > 64 * 1024) {
-        set_error("bin transpose needs %zu bytes of LDS", lds_t);
-        return LBT_ERR_UNSUPPORTED;
-      }
+      dim3 grid(blocks(N, kTransRows), hs.n_groups);
       if (hs.bin_bytes == 1)
-        transpose_bins_kernel<uint8_t><<<grid, kThreads, lds_t, stream>>>(
-          static_cast<const uint8_t*>(hs.binned), hs.bin_offset, hs.bin_pitch, N, F, L.bins_t_stride,
+        transpose_bins_kernel<uint8_t><<<grid, kThreads, 0, stream>>>(
+          static_cast<const uint8_t*>(hs.binned), hs.groups, hs.bin_base, hs.bin_stride, N, L.bins_t_stride,
           static_cast<uint8_t*>(L.bins_t));
       else
-        transpose_bins_kernel<uint16_t><<<grid, kThreads, lds_t, stream>>>(
-          static_cast<const uint16_t*>(hs.binned), hs.bin_offset, hs.bin_pitch, N, F, L.bins_t_stride,
+        transpose_bins_kernel<uint16_t><<<grid, kThreads, 0, stream>>>(
+          static_cast<const uint16_t*>(hs.binned), hs.groups, hs.bin_base, hs.bin_stride, N, L.bins_t_stride,
           static_cast<uint16_t*>(L.bins_t));
     }
     if (depth < max_depth - 1) {
@@ -1285,10 +1284,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     auto& acc = profiler().acc;
     const bool cached = hs.binned != nullptr;
     for (int d = 0; d < max_depth && d < 64; d++) {
-      // bytes of one feature value as the level reads it (X itself, or its cached bin),
-      // plus the bins the root pass writes
-      double per_value = (cached && d > 0) ? hs.bin_bytes : static_cast<double>(sizeof(T));
-      if (cached && d == 0) per_value += hs.bin_bytes;
+      // bytes of one feature value as the level reads it (X itself, or its cached bin)
+      double per_value = cached ? hs.bin_bytes : static_cast<double>(sizeof(T));
       double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * per_value + K * 8.0 + 8.0) +
                   static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
       acc.level_bytes[d] += by;

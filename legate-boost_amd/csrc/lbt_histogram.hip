@@ -45,7 +45,22 @@ constexpr int kSmallNodeRows = 64;  // below this a node goes straight to global
 constexpr int kUnroll        = 4;   // rows per lane and tile, search kernel
 constexpr int kBinnedUnroll  = 8;   // rows per lane and tile, binned kernel
 constexpr int kLinearProbes  = 4;   // forward probes before falling back to a binary search
-constexpr size_t kLdsBudget  = 160 * 1024 - 512;
+constexpr size_t kLdsBudget  = 160 * 1024 - 512 - 4096;  // 4 KB stay free for the tile window
+#ifndef LBT_V_DEFER
+#define LBT_V_DEFER 1
+#endif
+#ifndef LBT_V_IDENT
+#define LBT_V_IDENT 1
+#endif
+#ifndef LBT_V_QUAD
+#define LBT_V_QUAD 0
+#endif
+#ifndef LBT_V_ABL
+#define LBT_V_ABL 0
+#endif
+#ifndef LBT_V_PROBES
+#define LBT_V_PROBES 8
+#endif
 
 // For the nodes [j0, j1) of the current level (level-local indices): decides
 // which are built (build_tree.h:92-104) and cuts their row segments into tiles
@@ -108,6 +123,29 @@ __global__ void __launch_bounds__(kPlanThreads)
     level_total->built_instances += s_rc;
     level_total->built_nodes += s_nb;
   }
+}
+
+// One descriptor per tile, so that the histogram kernels need no search while they walk:
+// (node, first row, end row, rows of the node), indexed like the tiles.
+__global__ void __launch_bounds__(kPlanThreads)
+  expand_tiles_kernel(int j0, int n_nodes, int level_first, const int32_t* seg, const int32_t* tile_start,
+                      const LevelMeta* meta, int tile_rows, int4* tiles)
+{
+  const int tile = blockIdx.x * kPlanThreads + threadIdx.x;
+  if (tile >= meta->n_tiles) return;
+  // last j with tile_start[j] <= tile
+  int lo = 0, hi = n_nodes;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (tile_start[mid] <= tile)
+      lo = mid;
+    else
+      hi = mid - 1;
+  }
+  const int j      = j0 + lo;
+  const int seg_lo = seg[j], seg_hi = seg[j + 1];
+  const int r0     = seg_lo + (tile - tile_start[lo]) * tile_rows;
+  tiles[tile]      = make_int4(level_first + j, r0, min(seg_hi, r0 + tile_rows), seg_hi - seg_lo);
 }
 
 // The cell of a value: monotone non-decreasing in x for any lo and invw >= 0
@@ -176,19 +214,22 @@ __global__ void __launch_bounds__(256)
 
 // What both kernels need to walk the tiles of a batch.
 struct TileWalk {
-  const int2* positions;  // (node,row) sorted by node
-  const int32_t* seg;     // level-local segment starts
-  int j0;                 // first level-local node of the batch
-  int n_nodes;            // nodes in the batch
-  int level_first;        // global index of level-local node 0
-  const int32_t* tile_start;
-  const LevelMeta* meta;
+  int j0;           // first level-local node of the batch
+  int n_nodes;      // nodes in the batch
+  int level_first;  // global index of level-local node 0
   int tile_rows;
   int rpp;       // rows per pass of a workgroup (tile_rows / rows per lane)
   int n_gk;      // groups * outputs
   int n_chunks;  // row-tile ranges
-  const unsigned long long* qstats;
 };
+
+// Read-only inputs of the tile walk. They are separate __restrict__ kernel
+// parameters (not struct members) so that the compiler can prove that no store of
+// the kernel touches them and fetch the uniform ones through the scalar cache;
+// vector loads here would force waits that also drain the prefetched row data.
+#define LBT_WALK_PARAMS                                                                 \
+  const int2* __restrict__ positions, const int4* __restrict__ tiles,                   \
+    const LevelMeta* __restrict__ meta, const unsigned long long* __restrict__ qstats
 
 struct Tile {
   int node;
@@ -196,47 +237,42 @@ struct Tile {
   int seg_rows;
 };
 
-// Node and row range of a tile. `hint` is the batch-local node of the previous
-// lookup (tiles are visited in order, so the node index only moves forward); a
-// negative hint starts with a binary search. All values are uniform over the
-// workgroup.
-__device__ inline Tile tile_lookup(const TileWalk& w, int tile, int& hint)
-{
-  int lo;
-  if (hint < 0) {
-    // last j with tile_start[j] <= tile
-    lo     = 0;
-    int hi = w.n_nodes;
-    while (lo < hi) {
-      int mid = (lo + hi + 1) >> 1;
-      if (w.tile_start[mid] <= tile)
-        lo = mid;
-      else
-        hi = mid - 1;
-    }
-  } else {
-    lo = hint;
-    while (w.tile_start[lo + 1] <= tile) lo++;
+// The workgroup keeps a window of tile descriptors in LDS and refills it when the walk
+// runs past its end; reading a descriptor is then an LDS access, not a chain of dependent
+// global loads that would stall every wave of the workgroup at the same time.
+constexpr int kTileWindow = 256;
+
+struct TileWindow {
+  int4* s_tiles;
+  const int4* tiles;
+  int base;
+  int t_end;
+  __device__ void fill(int first)
+  {
+    base = first;
+    __syncthreads();
+    for (int i = threadIdx.x; i < kTileWindow && first + i < t_end; i += blockDim.x) s_tiles[i] = tiles[first + i];
+    __syncthreads();
   }
-  hint             = lo;
-  const int j      = w.j0 + lo;
-  const int seg_lo = w.seg[j];
-  const int seg_hi = w.seg[j + 1];
-  Tile t;
-  t.node     = w.level_first + j;
-  t.r0       = seg_lo + (tile - w.tile_start[lo]) * w.tile_rows;
-  t.r1       = min(seg_hi, t.r0 + w.tile_rows);
-  t.seg_rows = seg_hi - seg_lo;
-  return t;
-}
+  // all threads of the workgroup call this with the same, non-decreasing tile index
+  __device__ Tile get(int tile)
+  {
+    if (tile - base >= kTileWindow) fill(tile);
+    const int4 d = s_tiles[tile - base];
+    Tile t;
+    t.node     = d.x;
+    t.r0       = d.y;
+    t.r1       = d.z;
+    t.seg_rows = d.w;
+    return t;
+  }
+};
 
 template <typename T>
 struct HistArgs {
   TileWalk w;
-  const T* X;
   int F;
   int64_t n_rows;
-  const int2* qgh;  // [N][K] packed int32 (grad, hess)
   int K;
   const T* proposals;
   const int32_t* row_pointers;
@@ -247,9 +283,6 @@ struct HistArgs {
   int cells;
   int search_steps;
   HistView hist;
-  void* binned;               // bin cache, written when kWriteBins
-  const int32_t* bin_offset;  // [F] element offset of a feature inside a cache row
-  int bin_pitch;              // elements per cache row
 };
 
 template <typename T, int VEC>
@@ -305,8 +338,9 @@ __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I
   }
 }
 
-template <typename T, int VEC, typename BinT, bool kWriteBins>
-__global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
+template <typename T, int VEC, bool kIdentityRows>
+__global__ void __launch_bounds__(kHistThreads)
+  histogram_kernel(HistArgs<T> a, LBT_WALK_PARAMS, const T* __restrict__ X, const int2* __restrict__ qgh)
 {
   using Vec = typename VecOf<T, VEC>::type;
   extern __shared__ unsigned char smem_raw[];
@@ -362,13 +396,9 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
     c_end[v]  = a.row_pointers[f + 1] - bin0;
   }
   const T cmax = static_cast<T>(C - 1);
-  const unsigned long long max_abs = w.qstats[0];
-  // unused elements between this group's sliver and the next one in a cache row
-  const int pad = kWriteBins ? (f1 < a.F ? a.bin_offset[f1] : a.bin_pitch) - (a.bin_offset[f0] + gs) : 0;
-  // this lane's place in a row of the bin cache
-  BinT* const bin_base = kWriteBins ? static_cast<BinT*>(a.binned) + a.bin_offset[min(f0 + fl, f1 - 1)] : nullptr;
+  const unsigned long long max_abs = qstats[0];
 
-  const int n_tiles = w.meta->n_tiles;
+  const int n_tiles = meta->n_tiles;
   const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
   const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / w.n_chunks);
 
@@ -376,50 +406,68 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
   unsigned long long acc = 0;  // rows added to the LDS copy since it was last merged
   __syncthreads();
 
-  auto load_rows = [&](const Tile& t, int (&row)[kUnroll]) {
+  // Loads are unconditional (an index past the tile is clamped to the tile's first row and
+  // the row is marked -1 afterwards), so that they issue back to back without branches.
+  // The loaded index is not looked at until the data loads of the following iteration, so
+  // nothing waits on it here; which rows of the tile exist is kept apart as a bit mask.
+  auto load_rows = [&](const Tile& t, int (&row)[kUnroll]) -> unsigned {
+    unsigned valid = 0;
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      int rr = t.r0 + rsub + u * w.rpp;
-      row[u] = (active && rr < t.r1) ? w.positions[rr].y : -1;
+      const int rr  = t.r0 + rsub + u * w.rpp;
+      const bool ok = active && rr < t.r1;
+      // at the root the order is still the identity: sorted index == row
+      if constexpr (kIdentityRows && LBT_V_IDENT)
+        row[u] = ok ? rr : t.r0;
+      else
+        row[u] = positions[ok ? rr : t.r0].y;
+#if !LBT_V_DEFER
+      row[u] = ok ? row[u] : -1;
+      if (row[u] < 0) row[u] = 0;
+#endif
+      valid |= ok ? (1u << u) : 0u;
     }
+    return valid;
   };
   auto load_data = [&](const int (&row)[kUnroll], Vec (&xv)[kUnroll], int2 (&q)[kUnroll]) {
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      if (row[u] >= 0) {
-        const T* xp = a.X + static_cast<int64_t>(row[u]) * a.F + (f0 + fl);
-        if constexpr (VEC == 1)
-          xv[u] = *xp;
-        else
-          xv[u] = *reinterpret_cast<const Vec*>(xp);
-        q[u] = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
-      }
+      const int64_t rw = row[u];
+      const T* xp      = X + rw * a.F + (f0 + fl);
+      if constexpr (VEC == 1)
+        xv[u] = *xp;
+      else
+        xv[u] = *reinterpret_cast<const Vec*>(xp);
+      q[u] = qgh[rw * a.K + k];
     }
   };
 
+  __shared__ int4 s_tile_window[kTileWindow];
+  TileWindow win{s_tile_window, tiles, 0, t_end};
+  win.fill(t_begin);
   Tile tc{}, tn{}, tnn{};
-  int hint = -1;
   int row_c[kUnroll], row_n[kUnroll], row_nn[kUnroll];
   Vec x_c[kUnroll], x_n[kUnroll];
   int2 q_c[kUnroll], q_n[kUnroll];
+  unsigned valid_c = 0, valid_n = 0, valid_nn = 0;
 #pragma unroll
-  for (int u = 0; u < kUnroll; u++) row_c[u] = row_n[u] = row_nn[u] = -1;
+  for (int u = 0; u < kUnroll; u++) row_c[u] = row_n[u] = row_nn[u] = 0;
   if (t_begin < t_end) {
-    tc = tile_lookup(w, t_begin, hint);
-    load_rows(tc, row_c);
+    tc      = win.get(t_begin);
+    valid_c = load_rows(tc, row_c);
     load_data(row_c, x_c, q_c);
   }
   if (t_begin + 1 < t_end) {
-    tn = tile_lookup(w, t_begin + 1, hint);
-    load_rows(tn, row_n);
+    tn      = win.get(t_begin + 1);
+    valid_n = load_rows(tn, row_n);
   }
 
   for (int tile = t_begin; tile < t_end; tile++) {
     // issue the loads of the next tile and the row indices of the one after
     if (tile + 1 < t_end) load_data(row_n, x_n, q_n);
     if (tile + 2 < t_end) {
-      tnn = tile_lookup(w, tile + 2, hint);
-      load_rows(tnn, row_nn);
+      tnn      = win.get(tile + 2);
+      valid_nn = load_rows(tnn, row_nn);
     }
 
     const int nrows   = tc.r1 - tc.r0;
@@ -438,10 +486,219 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
     I64Pair* gdst = a.hist.at(tc.node, k, bin0);
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      if (row_c[u] >= 0) {
+      if (valid_c & (1u << u)) {
         const unsigned long long packed =
           (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
           static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+        T xs[VEC];
+        if constexpr (VEC == 1) {
+          xs[0] = x_c[u];
+        } else if constexpr (VEC == 2) {
+          xs[0] = x_c[u].x;
+          xs[1] = x_c[u].y;
+        } else {
+          xs[0] = x_c[u].x;
+          xs[1] = x_c[u].y;
+          xs[2] = x_c[u].z;
+          xs[3] = x_c[u].w;
+        }
+#if LBT_V_QUAD
+        // The VEC searches of a lane advance together: their table lookups and each round of
+        // probes are issued back to back, and the wave leaves the loop when no lane has a
+        // proposal below its value left. A probe of a finished search is harmless (it fails).
+        int bin[VEC];
+        bool lt[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; v++)
+          bin[v] = c_prop[v] + s_cell[c_cell[v] + cell_of(xs[v], c_lo[v], c_invw[v], cmax)];
+        bool any_lt = false;
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+          lt[v] = s_prop[bin[v]] < xs[v];
+          any_lt |= lt[v];
+        }
+        int probes = 0;
+        while (__any(any_lt)) {
+#pragma unroll
+          for (int v = 0; v < VEC; v++) bin[v] += lt[v] ? 1 : 0;
+          if (++probes == kLinearProbes) {
+            // crowded cell: finish with a binary search over the rest of the feature
+#pragma unroll
+            for (int v = 0; v < VEC; v++)
+              bin[v] += count_less(s_prop + bin[v], c_end[v] - bin[v], xs[v], a.search_steps);
+            break;
+          }
+          any_lt = false;
+#pragma unroll
+          for (int v = 0; v < VEC; v++) {
+            lt[v] = s_prop[bin[v]] < xs[v];
+            any_lt |= lt[v];
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+          if (direct) {
+            atomic_add_i64(&gdst[bin[v]].grad, static_cast<int64_t>(q_c[u].x));
+            atomic_add_i64(&gdst[bin[v]].hess, static_cast<int64_t>(q_c[u].y));
+          } else {
+            atomicAdd(&s_hist[bin[v]], packed);
+          }
+        }
+#else
+        int bin[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+          const T x = xs[v];
+#if LBT_V_ABL & 8
+          int bn = c_prop[v] + (static_cast<int>(x * T(64)) & 63);
+#else
+          int bn = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+#endif
+#if !(LBT_V_ABL & 2)
+          bool lt    = s_prop[bn] < x;
+          int probes = 0;
+          while (__any(lt)) {
+            bn += lt ? 1 : 0;
+            if (++probes == kLinearProbes) {
+              bn += count_less(s_prop + bn, c_end[v] - bn, x, a.search_steps);
+              break;
+            }
+            lt = s_prop[bn] < x;
+          }
+#endif
+          bin[v] = bn;
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+#if !(LBT_V_ABL & 1)
+          if (direct) {
+            atomic_add_i64(&gdst[bin[v]].grad, static_cast<int64_t>(q_c[u].x));
+            atomic_add_i64(&gdst[bin[v]].hess, static_cast<int64_t>(q_c[u].y));
+          } else {
+            atomicAdd(&s_hist[bin[v]], packed);
+          }
+#else
+          if (bin[v] == -12345) s_hist[0] = packed;
+#endif
+        }
+#endif
+      }
+    }
+    // rotate the pipeline
+    tc      = tn;
+    tn      = tnn;
+    valid_c = valid_n;
+    valid_n = valid_nn;
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      row_c[u] = row_n[u];
+      row_n[u] = row_nn[u];
+      x_c[u]   = x_n[u];
+      q_c[u]   = q_n[u];
+    }
+  }
+  __syncthreads();
+  if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
+}
+
+// Root pass when the bin cache is in use: bins every value of X once and stores
+// the feature-relative bins, [row][feature], padded per group as described in
+// hist_prepare. No histogram is kept here, so the LDS holds only proposals and
+// lookup tables and a workgroup can cover all features of a row (100 features:
+// one group): X is then read and the cache written in whole, contiguous rows.
+// The root histogram itself is accumulated from the cache like every other
+// level.
+template <typename T>
+struct BinRowsArgs {
+  int F;
+  int64_t n_rows;
+  const T* proposals;
+  const int32_t* row_pointers;
+  const int32_t* groups;  // [n_groups+1]
+  const uint16_t* tables;
+  const T* cell_lo;
+  const T* cell_invw;
+  int cells;
+  int search_steps;
+  int n_groups;
+  int n_chunks;
+  int rpp;                    // rows per pass of a workgroup
+  const int64_t* bin_base;    // [F] element offset of a feature's bin of row 0 in the cache
+  const int32_t* bin_stride;  // [F] elements between consecutive rows
+};
+
+template <typename T, int VEC, typename BinT>
+__global__ void __launch_bounds__(kHistThreads)
+  bin_rows_kernel(BinRowsArgs<T> a, const T* __restrict__ X, BinT* __restrict__ binned)
+{
+  using Vec = typename VecOf<T, VEC>::type;
+  extern __shared__ unsigned char smem_raw[];
+  const int xcd   = blockIdx.x & 7;
+  const int slot  = blockIdx.x >> 3;
+  const int group = slot % a.n_groups;
+  const int chunk = (slot / a.n_groups) * 8 + xcd;
+  const int f0 = a.groups[group], f1 = a.groups[group + 1];
+  const int gs   = f1 - f0;
+  const int bin0 = a.row_pointers[f0];
+  const int nb   = a.row_pointers[f1] - bin0;
+  const int C    = a.cells;
+  T* s_prop        = reinterpret_cast<T*>(smem_raw);
+  uint16_t* s_cell = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(nb) * sizeof(T));
+  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_prop[i] = a.proposals[bin0 + i];
+  {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(a.tables + static_cast<int64_t>(f0) * C);
+    uint32_t* dst       = reinterpret_cast<uint32_t*>(s_cell);
+    const int words     = gs * C / 2;
+    for (int i = threadIdx.x; i < words; i += kHistThreads) dst[i] = src[i];
+  }
+  const int lanes_per_row = (gs + VEC - 1) / VEC;
+  const int lr            = threadIdx.x % lanes_per_row;
+  const int rsub          = threadIdx.x / lanes_per_row;
+  const bool active       = rsub < a.rpp;
+  const int fl            = lr * VEC;
+  T c_lo[VEC], c_invw[VEC];
+  int c_cell[VEC], c_prop[VEC], c_end[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; v++) {
+    int f     = min(f0 + fl + v, f1 - 1);
+    c_lo[v]   = a.cell_lo[f];
+    c_invw[v] = a.cell_invw[f];
+    c_cell[v] = (f - f0) * C;
+    c_prop[v] = a.row_pointers[f] - bin0;
+    c_end[v]  = a.row_pointers[f + 1] - bin0;
+  }
+  const T cmax  = static_cast<T>(C - 1);
+  const int pitch      = a.bin_stride[f0];
+  const int pad        = pitch - gs;  // unused elements behind the group's features in a cache row
+  BinT* const bin_base = binned + a.bin_base[min(f0 + fl, f1 - 1)];
+  const T* const x_base = X + (f0 + fl);
+  const int64_t r_begin = a.n_rows * chunk / a.n_chunks;
+  const int64_t r_end   = a.n_rows * (chunk + 1) / a.n_chunks;
+  __syncthreads();
+
+  // pass p covers rows r_begin + (p * kUnroll + u) * rpp + rsub; the values of the next pass
+  // are requested before the current one is searched
+  auto load_pass = [&](int64_t first, Vec (&xv)[kUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
+      r         = (active && r < r_end) ? r : r_begin;
+      const T* xp = x_base + r * a.F;
+      if constexpr (VEC == 1)
+        xv[u] = *xp;
+      else
+        xv[u] = *reinterpret_cast<const Vec*>(xp);
+    }
+  };
+  const int64_t pass_rows = static_cast<int64_t>(a.rpp) * kUnroll;
+  Vec x_c[kUnroll], x_n[kUnroll];
+  if (r_begin < r_end) load_pass(r_begin, x_c);
+  for (int64_t first = r_begin; first < r_end; first += pass_rows) {
+    if (first + pass_rows < r_end) load_pass(first + pass_rows, x_n);
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+      const int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
+      if (active && r < r_end) {
         T xs[VEC];
         if constexpr (VEC == 1) {
           xs[0] = x_c[u];
@@ -458,59 +715,39 @@ __global__ void __launch_bounds__(kHistThreads) histogram_kernel(HistArgs<T> a)
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
           const T x = xs[v];
-          int bin   = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
-          bool lt   = s_prop[bin] < x;
+          int bn    = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+          bool lt   = s_prop[bn] < x;
           int probes = 0;
           while (__any(lt)) {
-            bin += lt ? 1 : 0;
-            if (++probes == kLinearProbes) {
-              // crowded cell: finish with a binary search over the rest of the feature
-              bin += count_less(s_prop + bin, c_end[v] - bin, x, a.search_steps);
+            bn += lt ? 1 : 0;
+            if (++probes == LBT_V_PROBES) {
+              bn += count_less(s_prop + bn, c_end[v] - bn, x, a.search_steps);
               break;
             }
-            lt = s_prop[bin] < x;
+            lt = s_prop[bn] < x;
           }
-          rel[v] = static_cast<BinT>(bin - c_prop[v]);
-          if (direct) {
-            atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
-            atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
-          } else {
-            atomicAdd(&s_hist[bin], packed);
-          }
+          rel[v] = static_cast<BinT>(bn - c_prop[v]);
         }
-        if constexpr (kWriteBins) {
-          if (k == 0 && f0 + fl < f1) {
-            BinT* bp = bin_base + static_cast<int64_t>(row_c[u]) * a.bin_pitch;
-            if constexpr (VEC == 4 && sizeof(BinT) == 1) {
-              *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
-                                                 (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
-            } else {
+        if (f0 + fl < f1) {
+          BinT* bp = bin_base + r * pitch;
+          if constexpr (VEC == 4 && sizeof(BinT) == 1) {
+            *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
+                                               (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
+          } else {
 #pragma unroll
-              for (int v = 0; v < VEC; v++)
-                if (f0 + fl + v < f1) bp[v] = rel[v];
-            }
-            // the lane that holds the group's last features also clears the padding up to
-            // the next sliver, so that whole sectors are written
-            if (fl + VEC >= gs) {
-              for (int i = gs - fl; i < gs - fl + pad; i++) bp[i] = 0;
-            }
+            for (int v = 0; v < VEC; v++)
+              if (f0 + fl + v < f1) bp[v] = rel[v];
+          }
+          // the lane with the group's last features also clears the padding behind them
+          if (fl + VEC >= gs) {
+            for (int i = gs - fl; i < gs - fl + pad; i++) bp[i] = 0;
           }
         }
       }
     }
-    // rotate the pipeline
-    tc = tn;
-    tn = tnn;
 #pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
-      row_c[u] = row_n[u];
-      row_n[u] = row_nn[u];
-      x_c[u]   = x_n[u];
-      q_c[u]   = q_n[u];
-    }
+    for (int u = 0; u < kUnroll; u++) x_c[u] = x_n[u];
   }
-  __syncthreads();
-  if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
 }
 
 // Deeper levels: the bins of every (row, feature) are already known, so a lane
@@ -527,6 +764,10 @@ struct BinVec<uint16_t, 4> {
   using type = uint2;
 };
 template <>
+struct BinVec<uint8_t, 16> {
+  using type = uint4;
+};
+template <>
 struct BinVec<uint8_t, 1> {
   using type = uint8_t;
 };
@@ -540,6 +781,15 @@ __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int
 {
   if constexpr (BV == 1) {
     out[0] = w;
+  } else if constexpr (BV == 16) {
+    const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      out[4 * i + 0] = q[i] & 0xff;
+      out[4 * i + 1] = (q[i] >> 8) & 0xff;
+      out[4 * i + 2] = (q[i] >> 16) & 0xff;
+      out[4 * i + 3] = q[i] >> 24;
+    }
   } else if constexpr (sizeof(BinT) == 1) {
     out[0] = w & 0xff;
     out[1] = (w >> 8) & 0xff;
@@ -555,10 +805,8 @@ __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int
 
 struct BinnedArgs {
   TileWalk w;
-  const void* binned;
-  const int32_t* bin_offset;  // [F] element offset of a feature inside a cache row
-  int bin_pitch;              // elements per cache row
-  const int2* qgh;
+  const int64_t* bin_base;    // [F] element offset of a feature's bin of row 0 in the cache
+  const int32_t* bin_stride;  // [F] elements between consecutive rows
   int K;
   const int32_t* row_pointers;
   const int32_t* groups;
@@ -566,9 +814,12 @@ struct BinnedArgs {
 };
 
 template <typename BinT, int BV>
-__global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedArgs a)
+__global__ void __launch_bounds__(kHistThreads)
+  binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const BinT* __restrict__ binned,
+                          const int2* __restrict__ qgh)
 {
   using Word = typename BinVec<BinT, BV>::type;
+  constexpr int kRows = BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll;  // rows per lane and tile
   extern __shared__ unsigned char smem_raw[];
   const TileWalk& w = a.w;
   const int xcd   = blockIdx.x & 7;
@@ -582,7 +833,9 @@ __global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedAr
   const int bin0 = a.row_pointers[f0];
   const int nb   = a.row_pointers[f1] - bin0;
   unsigned long long* s_hist = reinterpret_cast<unsigned long long*>(smem_raw);
-  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_hist[i] = 0;
+  // behind the group's bins every lane owns a spare slot that takes the adds of its features
+  // past the group end (never read; private, so these adds do not collide)
+  for (int i = threadIdx.x; i < nb + kHistThreads; i += kHistThreads) s_hist[i] = 0;
 
   const int lanes_per_row = (gs + BV - 1) / BV;
   const int lr            = threadIdx.x % lanes_per_row;
@@ -590,58 +843,64 @@ __global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedAr
   const bool active       = rsub < w.rpp;
   const int fl            = lr * BV;
   const int f_lane        = min(f0 + fl, f1 - 1);
-  const BinT* const my_bins = static_cast<const BinT*>(a.binned) + a.bin_offset[f_lane];
-  const int my_stride       = a.bin_pitch;
+  const BinT* const my_bins = binned + a.bin_base[f_lane];
+  const int my_stride       = a.bin_stride[f_lane];
   int c_base[BV];
 #pragma unroll
-  for (int v = 0; v < BV; v++) c_base[v] = a.row_pointers[min(f0 + fl + v, f1 - 1)] - bin0;
-  const unsigned long long max_abs = w.qstats[0];
-  const int n_tiles = w.meta->n_tiles;
+  for (int v = 0; v < BV; v++) c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
+  const unsigned long long max_abs = qstats[0];
+  const int n_tiles = meta->n_tiles;
   const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
   const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / w.n_chunks);
   int cur_node           = -1;
   unsigned long long acc = 0;
   __syncthreads();
 
-  auto load_rows = [&](const Tile& t, int (&row)[kBinnedUnroll]) {
+  auto load_rows = [&](const Tile& t, int (&row)[kRows]) -> unsigned {
+    unsigned valid = 0;
 #pragma unroll
-    for (int u = 0; u < kBinnedUnroll; u++) {
-      int rr = t.r0 + rsub + u * w.rpp;
-      row[u] = (active && rr < t.r1) ? w.positions[rr].y : -1;
+    for (int u = 0; u < kRows; u++) {
+      const int rr  = t.r0 + rsub + u * w.rpp;
+      const bool ok = active && rr < t.r1;
+      row[u]        = positions[ok ? rr : t.r0].y;
+      valid |= ok ? (1u << u) : 0u;
     }
+    return valid;
   };
-  auto load_data = [&](const int (&row)[kBinnedUnroll], Word (&bw)[kBinnedUnroll], int2 (&q)[kBinnedUnroll]) {
+  auto load_data = [&](const int (&row)[kRows], Word (&bw)[kRows], int2 (&q)[kRows]) {
 #pragma unroll
-    for (int u = 0; u < kBinnedUnroll; u++) {
-      if (row[u] >= 0) {
-        bw[u] = *reinterpret_cast<const Word*>(my_bins + static_cast<int64_t>(row[u]) * my_stride);
-        q[u]  = a.qgh[static_cast<int64_t>(row[u]) * a.K + k];
-      }
+    for (int u = 0; u < kRows; u++) {
+      const int64_t rw = row[u];
+      bw[u]            = *reinterpret_cast<const Word*>(my_bins + rw * my_stride);
+      q[u]             = qgh[rw * a.K + k];
     }
   };
 
+  __shared__ int4 s_tile_window[kTileWindow];
+  TileWindow win{s_tile_window, tiles, 0, t_end};
+  win.fill(t_begin);
   Tile tc{}, tn{}, tnn{};
-  int hint = -1;
-  int row_c[kBinnedUnroll], row_n[kBinnedUnroll], row_nn[kBinnedUnroll];
-  Word b_c[kBinnedUnroll], b_n[kBinnedUnroll];
-  int2 q_c[kBinnedUnroll], q_n[kBinnedUnroll];
+  int row_c[kRows], row_n[kRows], row_nn[kRows];
+  Word b_c[kRows], b_n[kRows];
+  int2 q_c[kRows], q_n[kRows];
+  unsigned valid_c = 0, valid_n = 0, valid_nn = 0;
 #pragma unroll
-  for (int u = 0; u < kBinnedUnroll; u++) row_c[u] = row_n[u] = row_nn[u] = -1;
+  for (int u = 0; u < kRows; u++) row_c[u] = row_n[u] = row_nn[u] = 0;
   if (t_begin < t_end) {
-    tc = tile_lookup(w, t_begin, hint);
-    load_rows(tc, row_c);
+    tc      = win.get(t_begin);
+    valid_c = load_rows(tc, row_c);
     load_data(row_c, b_c, q_c);
   }
   if (t_begin + 1 < t_end) {
-    tn = tile_lookup(w, t_begin + 1, hint);
-    load_rows(tn, row_n);
+    tn      = win.get(t_begin + 1);
+    valid_n = load_rows(tn, row_n);
   }
 
   for (int tile = t_begin; tile < t_end; tile++) {
     if (tile + 1 < t_end) load_data(row_n, b_n, q_n);
     if (tile + 2 < t_end) {
-      tnn = tile_lookup(w, tile + 2, hint);
-      load_rows(tnn, row_nn);
+      tnn      = win.get(tile + 2);
+      valid_nn = load_rows(tnn, row_nn);
     }
     const int nrows   = tc.r1 - tc.r0;
     const bool direct = tc.seg_rows < kSmallNodeRows ||
@@ -656,33 +915,44 @@ __global__ void __launch_bounds__(kHistThreads) binned_histogram_kernel(BinnedAr
       }
       acc += nrows;
     }
-    I64Pair* gdst = a.hist.at(tc.node, k, bin0);
+    if (!direct) {
 #pragma unroll
-    for (int u = 0; u < kBinnedUnroll; u++) {
-      if (row_c[u] >= 0) {
-        const unsigned long long packed =
-          (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
-          static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
-        int rel[BV];
-        unpack_bins<BinT, BV>(b_c[u], rel);
+      for (int u = 0; u < kRows; u++) {
+        if (valid_c & (1u << u)) {
+          const unsigned long long packed =
+            (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
+            static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+          int rel[BV];
+          unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
-        for (int v = 0; v < BV; v++) {
-          if (fl + v < gs) {
-            const int bin = c_base[v] + rel[v];
-            if (direct) {
+          // features past the group end read the zeroed padding of the cache row: spare slot
+          for (int v = 0; v < BV; v++) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
+        }
+      }
+    } else {
+      I64Pair* gdst = a.hist.at(tc.node, k, bin0);
+#pragma unroll
+      for (int u = 0; u < kRows; u++) {
+        if (valid_c & (1u << u)) {
+          int rel[BV];
+          unpack_bins<BinT, BV>(b_c[u], rel);
+#pragma unroll
+          for (int v = 0; v < BV; v++) {
+            if (fl + v < gs) {
+              const int bin = c_base[v] + rel[v];
               atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
               atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
-            } else {
-              atomicAdd(&s_hist[bin], packed);
             }
           }
         }
       }
     }
-    tc = tn;
-    tn = tnn;
+    tc      = tn;
+    tn      = tnn;
+    valid_c = valid_n;
+    valid_n = valid_nn;
 #pragma unroll
-    for (int u = 0; u < kBinnedUnroll; u++) {
+    for (int u = 0; u < kRows; u++) {
       row_c[u] = row_n[u];
       row_n[u] = row_nn[u];
       b_c[u]   = b_n[u];
@@ -701,57 +971,77 @@ int allow_large_lds(KernelT kernel)
   return LBT_OK;
 }
 
-template <typename T, int VEC, typename BinT, bool kWriteBins>
-int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid)
+template <typename T, int VEC, bool kIdentityRows>
+int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, const HistBatch& b, unsigned grid)
 {
   static bool attr_set = false;
   if (!attr_set) {
-    LBT_TRY(allow_large_lds(histogram_kernel<T, VEC, BinT, kWriteBins>));
+    LBT_TRY(allow_large_lds(histogram_kernel<T, VEC, kIdentityRows>));
     attr_set = true;
   }
-  histogram_kernel<T, VEC, BinT, kWriteBins><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a);
+  histogram_kernel<T, VEC, kIdentityRows><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
+    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const T*>(b.X), b.qgh);
   return LBT_OK;
 }
 
 template <typename T, int VEC>
-int launch_search_bins(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, unsigned grid, bool write_bins)
+int launch_search_rows(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, const HistBatch& b,
+                       unsigned grid, bool identity)
 {
-  if (!write_bins) return launch_search<T, VEC, uint8_t, false>(stream, hs, a, grid);
-  if (hs.bin_bytes == 1) return launch_search<T, VEC, uint8_t, true>(stream, hs, a, grid);
-  return launch_search<T, VEC, uint16_t, true>(stream, hs, a, grid);
+  if (identity) return launch_search<T, VEC, true>(stream, hs, a, b, grid);
+  return launch_search<T, VEC, false>(stream, hs, a, b, grid);
+}
+
+template <typename T, int VEC, typename BinT>
+int launch_bin_rows(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
+{
+  static bool attr_set = false;
+  if (!attr_set) {
+    LBT_TRY(allow_large_lds(bin_rows_kernel<T, VEC, BinT>));
+    attr_set = true;
+  }
+  bin_rows_kernel<T, VEC, BinT><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a, static_cast<const T*>(b.X),
+                                                                            static_cast<BinT*>(hs.binned));
+  return LBT_OK;
+}
+
+template <typename T, int VEC>
+int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
+{
+  if (hs.bin_bytes == 1) return launch_bin_rows<T, VEC, uint8_t>(stream, hs, a, b, grid);
+  return launch_bin_rows<T, VEC, uint16_t>(stream, hs, a, b, grid);
 }
 
 template <typename BinT, int BV>
-int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, unsigned grid)
+int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
 {
   static bool attr_set = false;
   if (!attr_set) {
     LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV>));
     attr_set = true;
   }
-  binned_histogram_kernel<BinT, BV><<<grid, kHistThreads, hs.blds_bytes, stream>>>(a);
+  binned_histogram_kernel<BinT, BV><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
+    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const BinT*>(hs.binned), b.qgh);
   return LBT_OK;
 }
 
 // One resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD).
-int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_groups, int rpp, int unroll, unsigned* grid)
+int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_cu, int n_groups, int rpp, int unroll,
+              size_t lds_bytes, unsigned* grid)
 {
-  int device = 0, n_cu = 256;
-  LBT_HIP(hipGetDevice(&device));
-  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  w.positions   = b.positions;
-  w.seg         = b.seg;
+  (void)hs;
   w.j0          = b.j0;
   w.n_nodes     = b.n_nodes;
   w.level_first = b.level_first;
-  w.tile_start  = hs.tile_start;
-  w.meta        = hs.meta;
   w.rpp         = rpp;
   w.tile_rows   = rpp * unroll;
   w.n_gk        = n_groups * b.K;
-  w.qstats      = b.qstats;
   const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
-  int64_t per_xcd = std::max<int64_t>(1, (n_cu / 8) / w.n_gk);
+  const int per_cu = lds_bytes * 2 <= 160 * 1024 ? 2 : 1;
+#ifndef LBT_V_CUSUB
+#define LBT_V_CUSUB 0
+#endif
+  int64_t per_xcd  = std::max<int64_t>(1, (per_cu * (n_cu - LBT_V_CUSUB) / 8) / w.n_gk);
   per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
   w.n_chunks      = static_cast<int>(per_xcd * 8);
   *grid           = static_cast<unsigned>(per_xcd * 8 * w.n_gk);
@@ -761,39 +1051,79 @@ int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_groups
 template <typename T>
 int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, int depth)
 {
-  const bool use_cache = hs.binned != nullptr && depth > 0;
+  const bool use_cache = hs.binned != nullptr;
+  int device = 0, n_cu = 256;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+  if (use_cache && depth == 0) {
+    // fill the bin cache: one workgroup per CU, rows split evenly
+    ProfScope ps(LBT_PROF_BINNING, stream,
+                 static_cast<double>(b.n_rows) * b.F * (sizeof(T) + static_cast<double>(hs.bin_bytes)));
+    BinRowsArgs<T> a;
+    a.F            = b.F;
+    a.n_rows       = b.n_rows;
+    a.proposals    = static_cast<const T*>(b.proposals);
+    a.row_pointers = b.row_pointers;
+    a.groups       = hs.groups;
+    a.tables       = hs.tables;
+    a.cell_lo      = static_cast<const T*>(hs.cell_lo);
+    a.cell_invw    = static_cast<const T*>(hs.cell_invw);
+    a.cells        = hs.cells;
+    a.search_steps = hs.search_steps;
+    a.n_groups     = hs.n_groups;
+    a.rpp          = hs.rpp;
+    a.bin_base     = hs.bin_base;
+    a.bin_stride   = hs.bin_stride;
+    int64_t per_xcd = std::max<int64_t>(1, ((n_cu - LBT_V_CUSUB) / 8) / hs.n_groups);
+    per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (b.n_rows / (hs.rpp * kUnroll) + 7) / 8));
+    a.n_chunks      = static_cast<int>(per_xcd * 8);
+    const unsigned grid = static_cast<unsigned>(per_xcd * 8 * hs.n_groups);
+    int rc = LBT_OK;
+    if (hs.vec == 4) {
+      if constexpr (sizeof(T) == 4) rc = launch_bin_rows_t<T, 4>(stream, hs, a, b, grid);
+    } else if (hs.vec == 2) {
+      rc = launch_bin_rows_t<T, 2>(stream, hs, a, b, grid);
+    } else {
+      rc = launch_bin_rows_t<T, 1>(stream, hs, a, b, grid);
+    }
+    LBT_TRY(rc);
+  }
   TileWalk w;
   unsigned grid = 0;
-  LBT_TRY(fill_walk(w, hs, b, use_cache ? hs.n_bgroups : hs.n_groups, use_cache ? hs.brpp : hs.rpp,
-                    use_cache ? kBinnedUnroll : kUnroll, &grid));
+  LBT_TRY(fill_walk(w, hs, b, n_cu, hs.n_groups, use_cache ? hs.brpp : hs.rpp,
+                    use_cache ? (hs.bvec == 16 ? kBinnedUnroll / 2 : kBinnedUnroll) : kUnroll,
+                    use_cache ? hs.blds_bytes : hs.lds_bytes, &grid));
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
     plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
                                                       b.K, b.hist.node_begin, b.hist.node_end, w.tile_rows,
                                                       hs.tile_start, hs.meta, b.level_total);
+    const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
+    expand_tiles_kernel<<<static_cast<unsigned>((max_tiles + kPlanThreads - 1) / kPlanThreads), kPlanThreads, 0,
+                          stream>>>(b.j0, b.n_nodes, b.level_first, b.seg, hs.tile_start, hs.meta, w.tile_rows,
+                                    hs.tiles);
   }
   ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   if (use_cache) {
     BinnedArgs a;
     a.w            = w;
-    a.binned       = hs.binned;
-    a.bin_offset   = hs.bin_offset;
-    a.bin_pitch    = hs.bin_pitch;
-    a.qgh          = b.qgh;
+    a.bin_base     = hs.bin_base;
+    a.bin_stride   = hs.bin_stride;
     a.K            = b.K;
     a.row_pointers = b.row_pointers;
-    a.groups       = hs.bgroups;
+    a.groups       = hs.groups;
     a.hist         = b.hist;
+    if (hs.bin_bytes == 1 && hs.bvec == 16) return launch_binned<uint8_t, 16>(stream, hs, a, b, grid);
     if (hs.bin_bytes == 1)
-      return hs.bvec == 4 ? launch_binned<uint8_t, 4>(stream, hs, a, grid) : launch_binned<uint8_t, 1>(stream, hs, a, grid);
-    return hs.bvec == 4 ? launch_binned<uint16_t, 4>(stream, hs, a, grid) : launch_binned<uint16_t, 1>(stream, hs, a, grid);
+      return hs.bvec == 4 ? launch_binned<uint8_t, 4>(stream, hs, a, b, grid)
+                          : launch_binned<uint8_t, 1>(stream, hs, a, b, grid);
+    return hs.bvec == 4 ? launch_binned<uint16_t, 4>(stream, hs, a, b, grid)
+                        : launch_binned<uint16_t, 1>(stream, hs, a, b, grid);
   }
   HistArgs<T> a;
   a.w            = w;
-  a.X            = static_cast<const T*>(b.X);
   a.F            = b.F;
   a.n_rows       = b.n_rows;
-  a.qgh          = b.qgh;
   a.K            = b.K;
   a.proposals    = static_cast<const T*>(b.proposals);
   a.row_pointers = b.row_pointers;
@@ -804,21 +1134,17 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   a.cells        = hs.cells;
   a.search_steps = hs.search_steps;
   a.hist         = b.hist;
-  a.binned       = hs.binned;
-  a.bin_offset   = hs.bin_offset;
-  a.bin_pitch    = hs.bin_pitch;
-  const bool write_bins = hs.binned != nullptr && depth == 0;
   if (hs.vec == 4) {
-    if constexpr (sizeof(T) == 4) return launch_search_bins<T, 4>(stream, hs, a, grid, write_bins);
+    if constexpr (sizeof(T) == 4) return launch_search_rows<T, 4>(stream, hs, a, b, grid, depth == 0);
   }
-  if (hs.vec == 2) return launch_search_bins<T, 2>(stream, hs, a, grid, write_bins);
-  return launch_search_bins<T, 1>(stream, hs, a, grid, write_bins);
+  if (hs.vec == 2) return launch_search_rows<T, 2>(stream, hs, a, b, grid, depth == 0);
+  return launch_search_rows<T, 1>(stream, hs, a, b, grid, depth == 0);
 }
 
 // Packs consecutive features, `unit` at a time, into groups whose LDS need
 // (bytes_of(feature)) stays within the budget; a second pass balances widths.
 template <typename BytesOf>
-size_t pack_groups(int F, int unit, BytesOf bytes_of, std::vector<int32_t>& groups)
+size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_of, std::vector<int32_t>& groups)
 {
   const int max_lanes = kHistThreads / 2;  // at least two rows per pass
   size_t lds          = 0;
@@ -830,7 +1156,7 @@ size_t pack_groups(int F, int unit, BytesOf bytes_of, std::vector<int32_t>& grou
     for (int f = 0; f < F; f += unit) {
       size_t cb = 0;
       for (int i = f; i < std::min(F, f + unit); i++) cb += bytes_of(i);
-      if (width > 0 && (cur + cb > kLdsBudget || width + unit > target || (width + unit) / unit > max_lanes)) {
+      if (width > 0 && (cur + cb > budget || width + unit > target || (width + unit + lane_vec - 1) / lane_vec > max_lanes)) {
         groups.push_back(f);
         lds   = std::max(lds, cur);
         cur   = 0;
@@ -866,82 +1192,98 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t 
                  const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
                  const void* X)
 {
-  (void)n_rows;
   const size_t elem = is_f64 ? 8 : 4;
   hs.is_f64         = is_f64;
   hs.n_features     = F;
-  // widest aligned vector of features a lane can load
+  // widest aligned vector of features a lane can load from X
   int vec = is_f64 ? 2 : 4;
   while (vec > 1 && (F % vec != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0)) vec >>= 1;
-  hs.vec  = vec;
-  hs.bvec = (F % 4 == 0) ? 4 : 1;
-  // group boundaries suit both the search kernel and the cached-bin layout
-  const int unit = hs.binned != nullptr ? std::max(vec, hs.bvec) : vec;
+  hs.vec = vec;
   int max_feature_bins = 1;
   for (int f = 0; f < F; f++) max_feature_bins = std::max(max_feature_bins, rp[f + 1] - rp[f]);
   hs.search_steps = 0;
   while ((1 << hs.search_steps) < max_feature_bins + 1) hs.search_steps++;
+  const bool cached = hs.binned != nullptr;
+  hs.bin_bytes      = max_feature_bins <= 256 ? 1 : 2;
+  // cached bins a lane of the histogram kernel loads at once: 16 bytes of one-byte bins
+  hs.bvec = !cached ? 1 : (hs.bin_bytes == 1 ? 16 : 4);
+  const int unit = cached ? std::max(vec, hs.bvec) : vec;
 
-  // table size: four cells per proposal of the widest feature, within [64, kMaxCells]
-  int cells = 64;
-  while (cells < 4 * max_feature_bins && cells < kMaxCells) cells <<= 1;
+  // LDS a feature needs: the search side keeps proposals and a lookup table; the packed
+  // sub-histogram joins them unless the bins are cached (then the root pass only bins and the
+  // histogram kernel keeps nothing but the sub-histogram)
+  auto search_bytes = [&](int f, int cells) {
+    return static_cast<size_t>(rp[f + 1] - rp[f]) * (cached ? elem : 8 + elem) + static_cast<size_t>(cells) * 2;
+  };
+  auto hist_bytes = [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; };
   std::vector<int32_t> groups;
-  size_t lds = 0;
+  size_t budget = kLdsBudget;
+  size_t lds    = 0;
   for (;;) {
-    lds = pack_groups(F, unit, [&](int f) {
-      return static_cast<size_t>(rp[f + 1] - rp[f]) * (8 + elem) + static_cast<size_t>(cells) * 2;
-    }, groups);
-    if (lds <= kLdsBudget) break;
-    if (cells <= 64) {
-      set_error("a feature group does not fit the LDS (%zu bytes)", lds);
+    // groups as wide as the tighter of the two kernels allows, with the smallest table
+    lds = pack_groups(F, unit, cached ? std::min(vec, hs.bvec) : vec, budget - (cached ? 8 * kHistThreads : 0),
+                      [&](int f) { return std::max(search_bytes(f, 64), cached ? hist_bytes(f) : 0); },
+                      groups);
+    size_t need = 0;
+    for (size_t g = 0; g + 1 < groups.size(); g++) {
+      size_t sb = 0;
+      for (int f = groups[g]; f < groups[g + 1]; f++) sb += search_bytes(f, 64);
+      need = std::max(need, sb);
+    }
+    if (lds <= kLdsBudget && need <= kLdsBudget) break;
+    if (budget <= 16 * 1024) {
+      set_error("a feature group does not fit the LDS (%zu bytes)", std::max(lds, need));
       return LBT_ERR_UNSUPPORTED;
     }
-    cells >>= 1;
+    budget -= 16 * 1024;
+  }
+  // table size: the largest, up to four cells per proposal, that still fits these groups
+  int cells = 64;
+  size_t search_lds = 0;
+  for (int c = 64; c <= kMaxCells && c <= 4 * std::max(16, max_feature_bins); c <<= 1) {
+    size_t need = 0;
+    for (size_t g = 0; g + 1 < groups.size(); g++) {
+      size_t sb = 0;
+      for (int f = groups[g]; f < groups[g + 1]; f++) sb += search_bytes(f, c);
+      need = std::max(need, sb);
+    }
+    if (need > kLdsBudget) break;
+    cells      = c;
+    search_lds = need;
   }
   hs.cells     = cells;
   hs.n_groups  = static_cast<int>(groups.size()) - 1;
-  hs.lds_bytes = (lds + 15) & ~size_t(15);
+  hs.lds_bytes = (search_lds + 15) & ~size_t(15);
   hs.rpp       = rows_per_pass(groups, vec);
   LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
-  if (hs.binned != nullptr) {
-    hs.bin_bytes = max_feature_bins <= 256 ? 1 : 2;
-    // groups of the binned kernel: only the packed sub-histogram lives in LDS
-    std::vector<int32_t> bg;
-    size_t blds = pack_groups(F, hs.bvec, [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; }, bg);
-    if (blds > kLdsBudget) {
-      set_error("a feature's histogram does not fit the LDS (%zu bytes)", blds);
-      return LBT_ERR_UNSUPPORTED;
+  if (cached) {
+    size_t blds = 0;
+    for (size_t g = 0; g + 1 < groups.size(); g++) {
+      size_t hb = 0;
+      for (int f = groups[g]; f < groups[g + 1]; f++) hb += hist_bytes(f);
+      blds = std::max(blds, hb);
     }
-    hs.n_bgroups  = static_cast<int>(bg.size()) - 1;
-    hs.blds_bytes = (blds + 15) & ~size_t(15);
-    hs.brpp       = rows_per_pass(bg, hs.bvec);
-    LBT_HIP(hipMemcpyAsync(hs.bgroups, bg.data(), sizeof(int32_t) * bg.size(), hipMemcpyHostToDevice, stream));
-    // a cache row: the search groups' slivers one after another, each padded to `align`
-    // bytes (a 32-byte sector if the row budget allows, else less)
-    std::vector<int32_t> off(F);
-    for (int align = 32;; align >>= 1) {
-      int64_t at = 0;
-      for (size_t g = 0; g + 1 < groups.size(); g++) {
-        for (int f = groups[g]; f < groups[g + 1]; f++) off[f] = static_cast<int32_t>(at + (f - groups[g]));
-        int64_t bytes = static_cast<int64_t>(groups[g + 1] - groups[g]) * hs.bin_bytes;
-        bytes         = (bytes + align - 1) / align * align;
-        at += bytes / hs.bin_bytes;
+    hs.blds_bytes = (blds + 8 * kHistThreads + 15) & ~size_t(15);  // + one spare slot per lane
+    hs.brpp       = rows_per_pass(groups, hs.bvec);
+    // the cache: one array per group, [row][features of the group padded to 32 bytes]
+    std::vector<int64_t> base(F);
+    std::vector<int32_t> stride(F);
+    int64_t at = 0;
+    for (size_t g = 0; g + 1 < groups.size(); g++) {
+      const int gs        = groups[g + 1] - groups[g];
+      const int64_t pitch = (static_cast<int64_t>(gs) * hs.bin_bytes + 31) / 32 * 32 / hs.bin_bytes;
+      for (int f = groups[g]; f < groups[g + 1]; f++) {
+        base[f]   = at + (f - groups[g]);
+        stride[f] = static_cast<int32_t>(pitch);
       }
-      if (at * hs.bin_bytes <= bin_row_bytes_max(F, hs.bin_bytes) || align <= 4) {
-        hs.bin_pitch = static_cast<int>(at);
-        break;
-      }
+      at += n_rows * pitch;
     }
-    if (static_cast<int64_t>(hs.bin_pitch) * hs.bin_bytes > bin_row_bytes_max(F, hs.bin_bytes)) {
-      set_error("bin cache row of %d bytes exceeds the workspace share", hs.bin_pitch * hs.bin_bytes);
+    if (at * hs.bin_bytes > n_rows * bin_row_bytes_max(F, hs.bin_bytes)) {
+      set_error("bin cache of %lld bytes exceeds the workspace share", static_cast<long long>(at * hs.bin_bytes));
       return LBT_ERR_WORKSPACE;
     }
-    hs.trans_span = 0;
-    for (int fa = 0; fa < F; fa += kTransposeFeatures) {
-      int fb = std::min(F, fa + kTransposeFeatures);
-      hs.trans_span = std::max(hs.trans_span, off[fb - 1] + 1 - off[fa] / 4 * 4);
-    }
-    LBT_HIP(hipMemcpyAsync(hs.bin_offset, off.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
+    LBT_HIP(hipMemcpyAsync(hs.bin_base, base.data(), sizeof(int64_t) * F, hipMemcpyHostToDevice, stream));
+    LBT_HIP(hipMemcpyAsync(hs.bin_stride, stride.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
     // the host vectors must outlive the asynchronous copies
     LBT_HIP(hipStreamSynchronize(stream));
   }

@@ -272,24 +272,24 @@ struct HistSetup {
   void* cell_lo      = nullptr;  // X dtype [n_features]
   void* cell_invw    = nullptr;  // X dtype [n_features]
   int32_t* tile_start = nullptr;
+  int4* tiles         = nullptr;  // one descriptor per tile of the batch in flight
   LevelMeta* meta    = nullptr;
-  // bin cache: feature-relative bin of every (row, feature), written by the
-  // root-level pass and read by all deeper levels instead of X
-  void* binned         = nullptr;  // uint8 or uint16 [n_rows][n_features], or null (cache off)
+  // bin cache: feature-relative bin of every (row, feature), written by the root binning
+  // pass and read by the histogram kernel of every level instead of X. When it is in use the
+  // groups above serve both kernels and the cache is stored group by group:
+  // [group][row][features of the group, padded to a 32-byte sector].
+  void* binned         = nullptr;  // uint8 or uint16, or null (cache off)
   int bin_bytes        = 0;        // 1 or 2
-  int32_t* bgroups     = nullptr;  // feature groups of the binned kernel [n_bgroups + 1]
-  int n_bgroups        = 0;
-  int bvec             = 1;
-  size_t blds_bytes    = 0;
-  int32_t* bin_offset  = nullptr;  // [n_features] element offset of a feature inside a cache row
-  int bin_pitch        = 0;        // elements per cache row
-  int trans_span       = 0;        // widest stretch of a cache row that kTransposeFeatures features cover
-  int rpp              = 0;        // rows per workgroup pass, search kernel
-  int brpp             = 0;        // rows per workgroup pass, binned kernel
+  int bvec             = 1;        // cached bins a lane of the histogram kernel loads at once
+  size_t blds_bytes    = 0;        // LDS of the histogram kernel (packed sub-histogram only)
+  int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
+  int32_t* bin_stride  = nullptr;  // [n_features] elements between consecutive rows
+  int rpp              = 0;        // rows per workgroup pass, search / binning kernel
+  int brpp             = 0;        // rows per workgroup pass, histogram kernel on cached bins
 };
 
 constexpr int kMaxCells = 2048;
-constexpr int kTransposeFeatures = 64;  // features one workgroup of the bin transpose handles
+constexpr int kTransposeFeatures = 64;  // features the bin transpose stages at a time
 
 // Upper bound on the bytes of one row of the bin cache (features plus sector padding
 // between groups); the workspace reserves n_rows times this.

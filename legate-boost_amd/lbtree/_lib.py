@@ -7,13 +7,14 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SO_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "liblbtree.so")
+# LBTREE_SO selects another build of the same library (kernel tuning)
+SO_PATH = os.environ.get("LBTREE_SO") or os.path.join(os.path.dirname(_HERE), "csrc", "liblbtree.so")
 
 LBT_OK = 0
 LBT_F32 = 0
 LBT_F64 = 1
 LBT_MAX_SPLIT_SAMPLES = 2048
-PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "positions", "other", "predict"]
+PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "positions", "other", "predict", "binning"]
 
 
 class BuildParams(C.Structure):
@@ -53,9 +54,9 @@ class BuildTaps(C.Structure):
 
 class Profile(C.Structure):
     _fields_ = [
-        ("launches", C.c_int64 * 8),
-        ("ms", C.c_double * 8),
-        ("bytes", C.c_double * 8),
+        ("launches", C.c_int64 * 9),
+        ("ms", C.c_double * 9),
+        ("bytes", C.c_double * 9),
         ("n_levels", C.c_int32),
         ("level_ms", C.c_double * 64),
         ("level_bytes", C.c_double * 64),
