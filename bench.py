@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--reference-flow", action="store_true",
                     help="update the training predictions with a PredictTask per round (as the reference loop does) instead of the row->leaf map that BuildTreeTask can return")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 4 GiB device copy five times (to scale rocprofv3's FETCH_SIZE / "
+                         "WRITE_SIZE counters against a kernel of known traffic)")
     return ap.parse_args()
 
 
@@ -169,7 +172,7 @@ def bench_training(args):
     ]
     out = {
         "metric": "boosting rounds/sec + histogram HBM GB/s (% peak), 10M×100 depth 8" if cfg == 2
-        else "boosting rounds/sec + histogram HBM GB/s (% peak), %s" % name,
+        else "boosting rounds/sec + histogram HBM GB/s (%% peak), %s" % name,
         "value": args.steps / dt,
         "unit": "rounds/s",
         "n_gpus": 1,
@@ -267,8 +270,27 @@ def bench_predict(args):
     return out
 
 
+def copy_calibration():
+    import torch
+
+    n = 1 << 30
+    a = torch.empty(n, dtype=torch.float32, device="cuda").normal_()
+    b = torch.empty_like(a)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / 5
+    print(json.dumps({"copy_bytes_read": n * 4, "copy_bytes_written": n * 4, "ms": dt * 1e3,
+                      "GBps_read_plus_write": 2 * n * 4 / dt / 1e9}))
+
+
 def main():
     args = parse()
+    if args.copy_calibration:
+        copy_calibration()
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives are built)"
               % args.gpus, file=sys.stderr)
