@@ -900,9 +900,13 @@ struct Layout {
   int32_t* row_pointers;
   int32_t* bin_feature;
   int32_t* groups;
+  int32_t* sgroups;
   int64_t* bin_base;
   int32_t* bin_stride;
+  int32_t* bin_tail;
+  RecInfo* rec;
   void* binned;
+  size_t binned_bytes;
   uint16_t* tables;
   void* cell_lo;
   void* cell_invw;
@@ -957,10 +961,14 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.row_pointers = ar.take<int32_t>(F + 1);
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
   L.groups       = ar.take<int32_t>(F + 1);
+  L.sgroups      = ar.take<int32_t>(F + 1);
   L.bin_base     = ar.take<int64_t>(F);
   L.bin_stride   = ar.take<int32_t>(F);
+  L.bin_tail     = ar.take<int32_t>(F);
+  L.rec          = ar.take<RecInfo>(F);
   // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
-  L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(static_cast<size_t>(N) * bin_row_bytes_max(F, S <= 256 ? 1 : 2) + 16)) : nullptr;
+  L.binned_bytes = max_depth >= 2 ? static_cast<size_t>(N) * bin_row_bytes_max(F, S) : 0;
+  L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(L.binned_bytes + 16)) : nullptr;
   L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
   L.cell_lo      = ar.take<double>(F);
   L.cell_invw    = ar.take<double>(F);
@@ -1057,16 +1065,20 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
 
   HistSetup hs;
   hs.groups     = L.groups;
+  hs.sgroups    = L.sgroups;
   hs.tables     = L.tables;
   hs.cell_lo    = L.cell_lo;
   hs.cell_invw  = L.cell_invw;
   hs.tile_start = L.tile_start;
   hs.tiles      = L.tiles;
   hs.binned     = L.binned;
+  hs.binned_capacity = L.binned_bytes;
   hs.bin_base   = L.bin_base;
   hs.bin_stride = L.bin_stride;
+  hs.bin_tail   = L.bin_tail;
+  hs.rec        = L.rec;
   hs.meta       = L.meta;
-  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, N, rp, L.proposals, L.row_pointers, X));
+  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
 
   // ---- quantiser
   {
@@ -1161,7 +1173,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
         HistBatch hb;
         hb.X = X; hb.F = F; hb.qgh = L.qgh; hb.K = K; hb.positions = L.pos[cur_pos]; hb.seg = L.seg[cur_seg];
         hb.j0 = j0; hb.n_nodes = n_nodes; hb.level_first = level_first; hb.proposals = L.proposals;
-        hb.row_pointers = L.row_pointers; hb.hist = hv; hb.qstats = L.qstats; hb.node_sums = L.node_sums;
+        hb.row_pointers = L.row_pointers; hb.bin_feature = L.bin_feature; hb.hist = hv; hb.qstats = L.qstats; hb.node_sums = L.node_sums;
         hb.level_total = L.level_totals + depth; hb.n_rows = N;
         LBT_TRY(hist_launch(stream, hs, hb, depth));
       }

@@ -4,34 +4,36 @@
 // (rapidsai/legate-boost src/models/tree/build_tree.cu:213-577, build_tree.h:178-185).
 //
 // Layout of the work on gfx950:
-//   * Features are cut into groups whose state fits the LDS of one workgroup
-//     (160 KB): the group's proposals, a packed sub-histogram, and per feature a
-//     direct-lookup table from value to first reachable proposal.
-//   * A workgroup owns (a contiguous range of row tiles) x (group) x (output).
-//     All workgroups are resident at once; those that share a row range sit on
-//     the same XCD so that cache lines straddling two groups are fetched from
-//     HBM once.
-//   * A lane is tied to VEC consecutive features of its group and walks rows, so
-//     the lanes of a wave read consecutive bytes of a row with one 16-byte load
-//     each and keep their features' constants in registers. A tile is one pass of
-//     the workgroup (a few rows per lane); the loads of the next tile and the
-//     row indices of the one after are issued before the current tile is
-//     processed, so HBM latency hides behind the bin search.
-//   * Bin search: cell = clamp((x - lo) * invw) indexes the table, which gives the
-//     number of proposals in cells before it; a short forward probe over the
-//     proposals finishes the search. Any monotone cell function is exact here;
-//     the table is built on the device with the same function.
-//   * (grad, hess) of a row are one 64-bit word (grad in the high half, hess
-//     unsigned in the low half) added with a single LDS atomic; the sub-histogram
-//     is merged into the int64 histogram with global atomics when the workgroup
-//     moves to another node. Before the low half or the signed high half could
-//     overflow (rows * max |q| >= 2^31) the sub-histogram is merged early; rows of
-//     tiny nodes go straight to global atomics.
-//   * The root-level pass also stores the feature-relative bin of every value
-//     (one or two bytes). Deeper levels read those instead of X and skip the
-//     search. A cache row holds the groups' slivers one after another, each
-//     padded to a 32-byte sector (128 bytes per row for 100 features in four
-//     groups), so a row gathered at a deep level costs one cache line.
+//   * The lower bound of a value does not depend on the tree level, so it is
+//     computed once: a root pass (bin_rows_kernel) reads X in whole rows and
+//     stores the feature-relative bin of every value in one or two bytes (the
+//     bin cache). The histograms of all levels, the root included, are then
+//     accumulated from the cache (binned_histogram_kernel); a level reads a
+//     quarter of the bytes X would cost and does no search.
+//   * Bin search: cell = clamp((x - lo) * invw) indexes a per-feature table that
+//     gives the number of proposals in cells before it; a short forward probe over
+//     the proposals finishes the search. Any monotone cell function is exact
+//     here; the table is built on the device with the same function. Proposals
+//     and tables of a search group of features sit in LDS (all 100 features of a
+//     10M x 100 matrix with 256 proposals each are one group).
+//   * The packed sub-histogram of a histogram group of features (8 bytes per bin)
+//     is the only LDS state of the histogram kernel. (grad, hess) of a row are
+//     one 64-bit word (grad in the high half, hess unsigned in the low half)
+//     added with a single LDS atomic; the sub-histogram is merged into the int64
+//     histogram with global atomics when the workgroup moves to another node.
+//     Before the low half or the signed high half could overflow
+//     (rows * max |q| >= 2^31) it is merged early; rows of tiny nodes go
+//     straight to global atomics.
+//   * The cache is stored histogram group by histogram group, [group][row][record].
+//     A record holds the group's bins and, for single-output trees, the row's
+//     packed (grad, hess), padded to 32 bytes: 64 bytes for 52 features. A
+//     row gathered at a deep level then costs one cache line per group and the
+//     gradient pair comes with it instead of through a second gather.
+//   * A histogram workgroup owns (a contiguous range of row tiles) x (group) x
+//     (output). All workgroups are resident at once. A lane is tied to 16 bytes
+//     of the record and walks rows; a tile is one pass of the workgroup (a few
+//     rows per lane); the loads of the next tile and the row indices of the one
+//     after are issued before the current tile is processed.
 #include "lbt_internal.h"
 
 #include <algorithm>
@@ -40,27 +42,12 @@ namespace lbt {
 namespace {
 
 constexpr int kPlanThreads   = 256;
-constexpr int kHistThreads   = 1024;
 constexpr int kSmallNodeRows = 64;  // below this a node goes straight to global atomics
-constexpr int kUnroll        = 4;   // rows per lane and tile, search kernel
-constexpr int kBinnedUnroll  = 8;   // rows per lane and tile, binned kernel
-constexpr int kLinearProbes  = 4;   // forward probes before falling back to a binary search
-constexpr size_t kLdsBudget  = 160 * 1024 - 512 - 4096;  // 4 KB stay free for the tile window
-#ifndef LBT_V_DEFER
-#define LBT_V_DEFER 1
-#endif
-#ifndef LBT_V_IDENT
-#define LBT_V_IDENT 1
-#endif
-#ifndef LBT_V_QUAD
-#define LBT_V_QUAD 0
-#endif
-#ifndef LBT_V_ABL
-#define LBT_V_ABL 0
-#endif
-#ifndef LBT_V_PROBES
-#define LBT_V_PROBES 8
-#endif
+constexpr int kUnroll        = 4;   // rows per lane and tile, search kernels
+constexpr int kBinnedUnroll  = 8;   // rows per lane and tile, histogram kernel (halved for 16-byte loads)
+constexpr int kLinearProbes  = 8;   // forward probes before falling back to a binary search
+constexpr int kProbePad      = 3;   // +inf entries behind every feature's proposals in the binning pass
+constexpr int kProbeSlack    = 8;   // further entries behind the last feature that a probe window may touch
 
 // For the nodes [j0, j1) of the current level (level-local indices): decides
 // which are built (build_tree.h:92-104) and cuts their row segments into tiles
@@ -148,15 +135,21 @@ __global__ void __launch_bounds__(kPlanThreads)
   tiles[tile]      = make_int4(level_first + j, r0, min(seg_hi, r0 + tile_rows), seg_hi - seg_lo);
 }
 
-// The cell of a value: monotone non-decreasing in x for any lo and invw >= 0
-// (rounded subtraction, rounded multiplication by a non-negative constant and
-// clamping are all monotone; NaN goes to cell 0).
-template <typename T>
-__device__ inline int cell_of(T x, T lo, T invw, T cmax)
+// The cell of a value, t = x * invw + nlo clamped to [0, cmax]: monotone non-decreasing in x
+// for any nlo and invw >= 0 (a fused multiply-add rounds once, and rounding and clamping keep
+// order); NaN goes to cell 0. Table construction and lookup share this function, which is
+// all that exactness needs.
+__device__ inline int cell_of(float x, float nlo, float invw, float cmax)
 {
-  T t = (x - lo) * invw;
-  t   = t > T(0) ? t : T(0);  // false for NaN
-  t   = t < cmax ? t : cmax;
+  // the median of (t, 0, cmax) is the clamp; with a NaN operand the instruction returns the
+  // minimum of the others, 0
+  return static_cast<int>(__builtin_amdgcn_fmed3f(fmaf(x, invw, nlo), 0.0f, cmax));
+}
+__device__ inline int cell_of(double x, double nlo, double invw, double cmax)
+{
+  double t = fma(x, invw, nlo);
+  t        = t > 0.0 ? t : 0.0;  // false for NaN
+  t        = t < cmax ? t : cmax;
   return static_cast<int>(t);
 }
 
@@ -188,9 +181,12 @@ __global__ void __launch_bounds__(256)
         invw = T(0);
       }
     }
-    s_lo      = lo;
-    s_invw    = invw;
-    lo_out[f]   = lo;
+    // the kernels evaluate x * invw + nlo
+    T nlo = -lo * invw;
+    if (!(nlo == nlo)) nlo = T(0);
+    s_lo        = nlo;
+    s_invw      = invw;
+    lo_out[f]   = nlo;
     invw_out[f] = invw;
   }
   __syncthreads();
@@ -417,14 +413,10 @@ __global__ void __launch_bounds__(kHistThreads)
       const int rr  = t.r0 + rsub + u * w.rpp;
       const bool ok = active && rr < t.r1;
       // at the root the order is still the identity: sorted index == row
-      if constexpr (kIdentityRows && LBT_V_IDENT)
+      if constexpr (kIdentityRows)
         row[u] = ok ? rr : t.r0;
       else
         row[u] = positions[ok ? rr : t.r0].y;
-#if !LBT_V_DEFER
-      row[u] = ok ? row[u] : -1;
-      if (row[u] < 0) row[u] = 0;
-#endif
       valid |= ok ? (1u << u) : 0u;
     }
     return valid;
@@ -502,59 +494,11 @@ __global__ void __launch_bounds__(kHistThreads)
           xs[2] = x_c[u].z;
           xs[3] = x_c[u].w;
         }
-#if LBT_V_QUAD
-        // The VEC searches of a lane advance together: their table lookups and each round of
-        // probes are issued back to back, and the wave leaves the loop when no lane has a
-        // proposal below its value left. A probe of a finished search is harmless (it fails).
-        int bin[VEC];
-        bool lt[VEC];
-#pragma unroll
-        for (int v = 0; v < VEC; v++)
-          bin[v] = c_prop[v] + s_cell[c_cell[v] + cell_of(xs[v], c_lo[v], c_invw[v], cmax)];
-        bool any_lt = false;
-#pragma unroll
-        for (int v = 0; v < VEC; v++) {
-          lt[v] = s_prop[bin[v]] < xs[v];
-          any_lt |= lt[v];
-        }
-        int probes = 0;
-        while (__any(any_lt)) {
-#pragma unroll
-          for (int v = 0; v < VEC; v++) bin[v] += lt[v] ? 1 : 0;
-          if (++probes == kLinearProbes) {
-            // crowded cell: finish with a binary search over the rest of the feature
-#pragma unroll
-            for (int v = 0; v < VEC; v++)
-              bin[v] += count_less(s_prop + bin[v], c_end[v] - bin[v], xs[v], a.search_steps);
-            break;
-          }
-          any_lt = false;
-#pragma unroll
-          for (int v = 0; v < VEC; v++) {
-            lt[v] = s_prop[bin[v]] < xs[v];
-            any_lt |= lt[v];
-          }
-        }
-#pragma unroll
-        for (int v = 0; v < VEC; v++) {
-          if (direct) {
-            atomic_add_i64(&gdst[bin[v]].grad, static_cast<int64_t>(q_c[u].x));
-            atomic_add_i64(&gdst[bin[v]].hess, static_cast<int64_t>(q_c[u].y));
-          } else {
-            atomicAdd(&s_hist[bin[v]], packed);
-          }
-        }
-#else
         int bin[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
           const T x = xs[v];
-#if LBT_V_ABL & 8
-          int bn = c_prop[v] + (static_cast<int>(x * T(64)) & 63);
-#else
           int bn = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
-#endif
-#if !(LBT_V_ABL & 2)
           bool lt    = s_prop[bn] < x;
           int probes = 0;
           while (__any(lt)) {
@@ -565,23 +509,17 @@ __global__ void __launch_bounds__(kHistThreads)
             }
             lt = s_prop[bn] < x;
           }
-#endif
           bin[v] = bn;
         }
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
-#if !(LBT_V_ABL & 1)
           if (direct) {
             atomic_add_i64(&gdst[bin[v]].grad, static_cast<int64_t>(q_c[u].x));
             atomic_add_i64(&gdst[bin[v]].hess, static_cast<int64_t>(q_c[u].y));
           } else {
             atomicAdd(&s_hist[bin[v]], packed);
           }
-#else
-          if (bin[v] == -12345) s_hist[0] = packed;
-#endif
         }
-#endif
       }
     }
     // rotate the pipeline
@@ -602,76 +540,102 @@ __global__ void __launch_bounds__(kHistThreads)
 }
 
 // Root pass when the bin cache is in use: bins every value of X once and stores
-// the feature-relative bins, [row][feature], padded per group as described in
-// hist_prepare. No histogram is kept here, so the LDS holds only proposals and
-// lookup tables and a workgroup can cover all features of a row (100 features:
-// one group): X is then read and the cache written in whole, contiguous rows.
-// The root histogram itself is accumulated from the cache like every other
-// level.
+// the feature-relative bins in the cache records. No histogram is kept here, so
+// the LDS holds only proposals and lookup tables and a workgroup can cover all
+// features of a row (100 features with 256 proposals each: one search group): X
+// is then read in whole, contiguous rows. A lane bins VEC consecutive features,
+// which always belong to one histogram group; the lane that holds the last
+// features of a histogram group also writes the record's zero bytes and, for
+// single-output trees, the row's packed (grad, hess). The root histogram itself
+// is accumulated from the cache like every other level.
 template <typename T>
 struct BinRowsArgs {
   int F;
   int64_t n_rows;
   const T* proposals;
   const int32_t* row_pointers;
-  const int32_t* groups;  // [n_groups+1]
+  const int32_t* bin_feature;  // [bins] feature of every proposal
+  const int32_t* sgroups;      // search groups: [n_sgroups+1]
   const uint16_t* tables;
   const T* cell_lo;
   const T* cell_invw;
   int cells;
   int search_steps;
-  int n_groups;
+  int n_sgroups;
   int n_chunks;
   int rpp;                    // rows per pass of a workgroup
   const int64_t* bin_base;    // [F] element offset of a feature's bin of row 0 in the cache
   const int32_t* bin_stride;  // [F] elements between consecutive rows
+  const int32_t* bin_tail;    // [F] histogram group + 1 behind its last feature, else 0
+  const RecInfo* rec;         // [histogram groups]
 };
 
 template <typename T, int VEC, typename BinT>
 __global__ void __launch_bounds__(kHistThreads)
-  bin_rows_kernel(BinRowsArgs<T> a, const T* __restrict__ X, BinT* __restrict__ binned)
+  bin_rows_kernel(BinRowsArgs<T> a, const T* __restrict__ X, const int2* __restrict__ qgh,
+                  BinT* __restrict__ binned)
 {
   using Vec = typename VecOf<T, VEC>::type;
   extern __shared__ unsigned char smem_raw[];
   const int xcd   = blockIdx.x & 7;
   const int slot  = blockIdx.x >> 3;
-  const int group = slot % a.n_groups;
-  const int chunk = (slot / a.n_groups) * 8 + xcd;
-  const int f0 = a.groups[group], f1 = a.groups[group + 1];
+  const int group = slot % a.n_sgroups;
+  const int chunk = (slot / a.n_sgroups) * 8 + xcd;
+  const int f0 = a.sgroups[group], f1 = a.sgroups[group + 1];
   const int gs   = f1 - f0;
   const int bin0 = a.row_pointers[f0];
   const int nb   = a.row_pointers[f1] - bin0;
   const int C    = a.cells;
+  // LDS copy of the group's proposals: every feature is followed by kProbePad more +inf
+  // entries, so a window of probes that starts anywhere in a feature stays ascending
   T* s_prop        = reinterpret_cast<T*>(smem_raw);
-  uint16_t* s_cell = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(nb) * sizeof(T));
-  for (int i = threadIdx.x; i < nb; i += kHistThreads) s_prop[i] = a.proposals[bin0 + i];
+  const int np     = nb + kProbePad * gs + kProbeSlack;
+  uint16_t* s_cell = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(np) * sizeof(T));
+  for (int i = threadIdx.x; i < nb; i += kHistThreads)
+    s_prop[i + kProbePad * (a.bin_feature[bin0 + i] - f0)] = a.proposals[bin0 + i];
+  for (int i = threadIdx.x; i < kProbePad * gs + kProbeSlack; i += kHistThreads) {
+    const int f = min(i / kProbePad, gs - 1);  // the slack follows the last feature
+    s_prop[a.row_pointers[f0 + f + 1] - bin0 + kProbePad * f + (i - kProbePad * f)] = std::numeric_limits<T>::infinity();
+  }
   {
     const uint32_t* src = reinterpret_cast<const uint32_t*>(a.tables + static_cast<int64_t>(f0) * C);
     uint32_t* dst       = reinterpret_cast<uint32_t*>(s_cell);
     const int words     = gs * C / 2;
     for (int i = threadIdx.x; i < words; i += kHistThreads) dst[i] = src[i];
   }
-  const int lanes_per_row = (gs + VEC - 1) / VEC;
+  // group widths are multiples of VEC, so every lane owns VEC real features
+  const int lanes_per_row = gs / VEC;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
   const bool active       = rsub < a.rpp;
-  const int fl            = lr * VEC;
+  const int fb            = f0 + lr * VEC;  // first feature of this lane
   T c_lo[VEC], c_invw[VEC];
   int c_cell[VEC], c_prop[VEC], c_end[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; v++) {
-    int f     = min(f0 + fl + v, f1 - 1);
+    const int f = fb + v;
     c_lo[v]   = a.cell_lo[f];
     c_invw[v] = a.cell_invw[f];
     c_cell[v] = (f - f0) * C;
-    c_prop[v] = a.row_pointers[f] - bin0;
-    c_end[v]  = a.row_pointers[f + 1] - bin0;
+    c_prop[v] = a.row_pointers[f] - bin0 + kProbePad * (f - f0);
+    c_end[v]  = a.row_pointers[f + 1] - bin0 + kProbePad * (f - f0);
   }
-  const T cmax  = static_cast<T>(C - 1);
-  const int pitch      = a.bin_stride[f0];
-  const int pad        = pitch - gs;  // unused elements behind the group's features in a cache row
-  BinT* const bin_base = binned + a.bin_base[min(f0 + fl, f1 - 1)];
-  const T* const x_base = X + (f0 + fl);
+  const T cmax         = static_cast<T>(C - 1);
+  const int pitch      = a.bin_stride[fb];
+  BinT* const bin_base = binned + a.bin_base[fb];
+  // what this lane writes behind its own bins (byte offsets from its first bin)
+  const int tg = a.bin_tail[fb + VEC - 1];
+  int tz_from = 0, tz_to = 0, tq = -1;
+  bool tz_words = false;
+  if (tg > 0) {
+    const RecInfo ri = a.rec[tg - 1];
+    const int my_off = static_cast<int>(a.bin_base[fb] * static_cast<int64_t>(sizeof(BinT)) - ri.base);
+    tz_from          = ri.bins_end - my_off;
+    tz_to            = ri.zero_end - my_off;
+    tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
+    tz_words         = ((ri.bins_end | ri.zero_end) & 3) == 0;
+  }
+  const T* const x_base = X + fb;
   const int64_t r_begin = a.n_rows * chunk / a.n_chunks;
   const int64_t r_end   = a.n_rows * (chunk + 1) / a.n_chunks;
   __syncthreads();
@@ -692,9 +656,18 @@ __global__ void __launch_bounds__(kHistThreads)
   };
   const int64_t pass_rows = static_cast<int64_t>(a.rpp) * kUnroll;
   Vec x_c[kUnroll], x_n[kUnroll];
+  int2 q_c[kUnroll];
   if (r_begin < r_end) load_pass(r_begin, x_c);
   for (int64_t first = r_begin; first < r_end; first += pass_rows) {
     if (first + pass_rows < r_end) load_pass(first + pass_rows, x_n);
+    // the few lanes that copy gradient pairs fetch them now; the search below hides the latency
+    if (tq >= 0) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; u++) {
+        const int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
+        q_c[u]          = qgh[(active && r < r_end) ? r : r_begin];
+      }
+    }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
       const int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
@@ -712,36 +685,48 @@ __global__ void __launch_bounds__(kHistThreads)
           xs[3] = x_c[u].w;
         }
         BinT rel[VEC];
+        // the table gives the first proposal the value can reach; the proposals from there on
+        // are ascending, so the bin is that start plus the number of proposals below the value.
+        // Four of them are compared at once, without a branch; the (rare) lanes that saw four
+        // smaller proposals look at four more, and then finish with a binary search.
+        int bn[VEC], cnt[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
-          const T x = xs[v];
-          int bn    = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
-          bool lt   = s_prop[bn] < x;
-          int probes = 0;
-          while (__any(lt)) {
-            bn += lt ? 1 : 0;
-            if (++probes == LBT_V_PROBES) {
-              bn += count_less(s_prop + bn, c_end[v] - bn, x, a.search_steps);
-              break;
-            }
-            lt = s_prop[bn] < x;
-          }
-          rel[v] = static_cast<BinT>(bn - c_prop[v]);
+          const T x   = xs[v];
+          bn[v]       = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+          const T* pp = s_prop + bn[v];
+          cnt[v]      = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0) + (pp[3] < x ? 1 : 0);
         }
-        if (f0 + fl < f1) {
-          BinT* bp = bin_base + r * pitch;
-          if constexpr (VEC == 4 && sizeof(BinT) == 1) {
-            *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
-                                               (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
-          } else {
 #pragma unroll
-            for (int v = 0; v < VEC; v++)
-              if (f0 + fl + v < f1) bp[v] = rel[v];
+        for (int v = 0; v < VEC; v++) {
+          if (__any(cnt[v] == 4)) {
+            const T x   = xs[v];
+            const T* pp = s_prop + bn[v] + 4;
+            const int c2 = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0) + (pp[3] < x ? 1 : 0);
+            cnt[v] += cnt[v] == 4 ? c2 : 0;
+            if (__any(cnt[v] == 8)) {
+              const int left = cnt[v] == 8 ? c_end[v] - (bn[v] + 8) : 0;
+              cnt[v] += count_less(pp + 4, left, x, a.search_steps);
+            }
           }
-          // the lane with the group's last features also clears the padding behind them
-          if (fl + VEC >= gs) {
-            for (int i = gs - fl; i < gs - fl + pad; i++) bp[i] = 0;
+          rel[v] = static_cast<BinT>(bn[v] + cnt[v] - c_prop[v]);
+        }
+        BinT* bp = bin_base + r * pitch;
+        if constexpr (VEC == 4 && sizeof(BinT) == 1) {
+          *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
+                                             (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
+        } else {
+#pragma unroll
+          for (int v = 0; v < VEC; v++) bp[v] = rel[v];
+        }
+        if (tg > 0) {
+          unsigned char* tail = reinterpret_cast<unsigned char*>(bp);
+          if (tz_words) {
+            for (int i = tz_from; i < tz_to; i += 4) *reinterpret_cast<uint32_t*>(tail + i) = 0u;
+          } else {
+            for (int i = tz_from; i < tz_to; i++) tail[i] = 0;
           }
+          if (tq >= 0) *reinterpret_cast<int2*>(tail + tq) = q_c[u];
         }
       }
     }
@@ -750,15 +735,10 @@ __global__ void __launch_bounds__(kHistThreads)
   }
 }
 
-// Deeper levels: the bins of every (row, feature) are already known, so a lane
-// loads BV cached bins of its row with one load and only accumulates. The
-// sub-histogram is the only LDS state, which allows much wider feature groups.
+// Histogram of one level from the cached bins: a lane loads BV cached bins of its
+// row with one load and only accumulates.
 template <typename BinT, int BV>
 struct BinVec;
-template <>
-struct BinVec<uint8_t, 4> {
-  using type = uint32_t;
-};
 template <>
 struct BinVec<uint16_t, 4> {
   using type = uint2;
@@ -767,21 +747,11 @@ template <>
 struct BinVec<uint8_t, 16> {
   using type = uint4;
 };
-template <>
-struct BinVec<uint8_t, 1> {
-  using type = uint8_t;
-};
-template <>
-struct BinVec<uint16_t, 1> {
-  using type = uint16_t;
-};
 
 template <typename BinT, int BV>
 __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int (&out)[BV])
 {
-  if constexpr (BV == 1) {
-    out[0] = w;
-  } else if constexpr (BV == 16) {
+  if constexpr (BV == 16) {
     const uint32_t q[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -790,11 +760,6 @@ __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int
       out[4 * i + 2] = (q[i] >> 16) & 0xff;
       out[4 * i + 3] = q[i] >> 24;
     }
-  } else if constexpr (sizeof(BinT) == 1) {
-    out[0] = w & 0xff;
-    out[1] = (w >> 8) & 0xff;
-    out[2] = (w >> 16) & 0xff;
-    out[3] = w >> 24;
   } else {
     out[0] = w.x & 0xffff;
     out[1] = w.x >> 16;
@@ -805,17 +770,18 @@ __device__ inline void unpack_bins(const typename BinVec<BinT, BV>::type& w, int
 
 struct BinnedArgs {
   TileWalk w;
-  const int64_t* bin_base;    // [F] element offset of a feature's bin of row 0 in the cache
-  const int32_t* bin_stride;  // [F] elements between consecutive rows
+  const RecInfo* rec;  // [groups]
   int K;
   const int32_t* row_pointers;
   const int32_t* groups;
   HistView hist;
 };
 
-template <typename BinT, int BV>
+// kEmbed: the records carry the packed (grad, hess) of their row (single-output trees);
+// otherwise the pair of (row, output) is gathered from qgh.
+template <typename BinT, int BV, bool kEmbed>
 __global__ void __launch_bounds__(kHistThreads)
-  binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const BinT* __restrict__ binned,
+  binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
                           const int2* __restrict__ qgh)
 {
   using Word = typename BinVec<BinT, BV>::type;
@@ -837,14 +803,17 @@ __global__ void __launch_bounds__(kHistThreads)
   // past the group end (never read; private, so these adds do not collide)
   for (int i = threadIdx.x; i < nb + kHistThreads; i += kHistThreads) s_hist[i] = 0;
 
+  const RecInfo ri        = a.rec[group];
   const int lanes_per_row = (gs + BV - 1) / BV;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
   const bool active       = rsub < w.rpp;
   const int fl            = lr * BV;
-  const int f_lane        = min(f0 + fl, f1 - 1);
-  const BinT* const my_bins = binned + a.bin_base[f_lane];
-  const int my_stride       = a.bin_stride[f_lane];
+  const int my_off        = lr * static_cast<int>(sizeof(Word));
+  const unsigned char* const my_rec = cache + ri.base;
+  const int64_t stride              = ri.stride;
+  // the gradient pair may share the last 16 bytes a lane loads as bins: that lane blanks them
+  const bool strip = kEmbed && BV == 16 && ri.q_off >= my_off && ri.q_off < my_off + static_cast<int>(sizeof(Word));
   int c_base[BV];
 #pragma unroll
   for (int v = 0; v < BV; v++) c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
@@ -870,9 +839,13 @@ __global__ void __launch_bounds__(kHistThreads)
   auto load_data = [&](const int (&row)[kRows], Word (&bw)[kRows], int2 (&q)[kRows]) {
 #pragma unroll
     for (int u = 0; u < kRows; u++) {
-      const int64_t rw = row[u];
-      bw[u]            = *reinterpret_cast<const Word*>(my_bins + rw * my_stride);
-      q[u]             = qgh[rw * a.K + k];
+      const int64_t rw          = row[u];
+      const unsigned char* recp = my_rec + rw * stride;
+      bw[u]                     = *reinterpret_cast<const Word*>(recp + my_off);
+      if constexpr (kEmbed)
+        q[u] = *reinterpret_cast<const int2*>(recp + ri.q_off);
+      else
+        q[u] = qgh[rw * a.K + k];
     }
   };
 
@@ -915,6 +888,13 @@ __global__ void __launch_bounds__(kHistThreads)
       }
       acc += nrows;
     }
+    if constexpr (kEmbed && BV == 16) {
+#pragma unroll
+      for (int u = 0; u < kRows; u++) {
+        b_c[u].z = strip ? 0u : b_c[u].z;
+        b_c[u].w = strip ? 0u : b_c[u].w;
+      }
+    }
     if (!direct) {
 #pragma unroll
       for (int u = 0; u < kRows; u++) {
@@ -925,7 +905,7 @@ __global__ void __launch_bounds__(kHistThreads)
           int rel[BV];
           unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
-          // features past the group end read the zeroed padding of the cache row: spare slot
+          // features past the group end read zero bytes of the record: spare slot
           for (int v = 0; v < BV; v++) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
         }
       }
@@ -1000,7 +980,7 @@ int launch_bin_rows(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T
     LBT_TRY(allow_large_lds(bin_rows_kernel<T, VEC, BinT>));
     attr_set = true;
   }
-  bin_rows_kernel<T, VEC, BinT><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a, static_cast<const T*>(b.X),
+  bin_rows_kernel<T, VEC, BinT><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a, static_cast<const T*>(b.X), b.qgh,
                                                                             static_cast<BinT*>(hs.binned));
   return LBT_OK;
 }
@@ -1012,24 +992,24 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
   return launch_bin_rows<T, VEC, uint16_t>(stream, hs, a, b, grid);
 }
 
-template <typename BinT, int BV>
+template <typename BinT, int BV, bool kEmbed>
 int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
 {
   static bool attr_set = false;
   if (!attr_set) {
-    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV>));
+    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV, kEmbed>));
     attr_set = true;
   }
-  binned_histogram_kernel<BinT, BV><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
-    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const BinT*>(hs.binned), b.qgh);
+  binned_histogram_kernel<BinT, BV, kEmbed><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
+    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh);
   return LBT_OK;
 }
 
-// One resident workgroup per CU; row-tile ranges come in multiples of 8 (one per XCD).
-int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_cu, int n_groups, int rpp, int unroll,
-              size_t lds_bytes, unsigned* grid)
+// As many resident workgroups as the LDS allows per CU; row-tile ranges come in multiples
+// of 8 (one per XCD).
+int fill_walk(TileWalk& w, const HistBatch& b, int n_cu, int n_groups, int rpp, int unroll, size_t lds_bytes,
+              unsigned* grid)
 {
-  (void)hs;
   w.j0          = b.j0;
   w.n_nodes     = b.n_nodes;
   w.level_first = b.level_first;
@@ -1038,10 +1018,7 @@ int fill_walk(TileWalk& w, const HistSetup& hs, const HistBatch& b, int n_cu, in
   w.n_gk        = n_groups * b.K;
   const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
   const int per_cu = lds_bytes * 2 <= 160 * 1024 ? 2 : 1;
-#ifndef LBT_V_CUSUB
-#define LBT_V_CUSUB 0
-#endif
-  int64_t per_xcd  = std::max<int64_t>(1, (per_cu * (n_cu - LBT_V_CUSUB) / 8) / w.n_gk);
+  int64_t per_xcd  = std::max<int64_t>(1, (per_cu * n_cu / 8) / w.n_gk);
   per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
   w.n_chunks      = static_cast<int>(per_xcd * 8);
   *grid           = static_cast<unsigned>(per_xcd * 8 * w.n_gk);
@@ -1056,7 +1033,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   LBT_HIP(hipGetDevice(&device));
   LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
   if (use_cache && depth == 0) {
-    // fill the bin cache: one workgroup per CU, rows split evenly
+    // fill the bin cache: rows split evenly over as many workgroups as are resident at once
     ProfScope ps(LBT_PROF_BINNING, stream,
                  static_cast<double>(b.n_rows) * b.F * (sizeof(T) + static_cast<double>(hs.bin_bytes)));
     BinRowsArgs<T> a;
@@ -1064,20 +1041,24 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     a.n_rows       = b.n_rows;
     a.proposals    = static_cast<const T*>(b.proposals);
     a.row_pointers = b.row_pointers;
-    a.groups       = hs.groups;
+    a.bin_feature  = b.bin_feature;
+    a.sgroups      = hs.sgroups;
     a.tables       = hs.tables;
     a.cell_lo      = static_cast<const T*>(hs.cell_lo);
     a.cell_invw    = static_cast<const T*>(hs.cell_invw);
     a.cells        = hs.cells;
     a.search_steps = hs.search_steps;
-    a.n_groups     = hs.n_groups;
+    a.n_sgroups    = hs.n_sgroups;
     a.rpp          = hs.rpp;
     a.bin_base     = hs.bin_base;
     a.bin_stride   = hs.bin_stride;
-    int64_t per_xcd = std::max<int64_t>(1, ((n_cu - LBT_V_CUSUB) / 8) / hs.n_groups);
-    per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (b.n_rows / (hs.rpp * kUnroll) + 7) / 8));
-    a.n_chunks      = static_cast<int>(per_xcd * 8);
-    const unsigned grid = static_cast<unsigned>(per_xcd * 8 * hs.n_groups);
+    a.bin_tail     = hs.bin_tail;
+    a.rec          = hs.rec;
+    const int per_cu = hs.lds_bytes * 2 <= 160 * 1024 ? 2 : 1;
+    int64_t per_xcd  = std::max<int64_t>(1, (per_cu * n_cu / 8) / hs.n_sgroups);
+    per_xcd          = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (b.n_rows / (hs.rpp * kUnroll) + 7) / 8));
+    a.n_chunks       = static_cast<int>(per_xcd * 8);
+    const unsigned grid = static_cast<unsigned>(per_xcd * 8 * hs.n_sgroups);
     int rc = LBT_OK;
     if (hs.vec == 4) {
       if constexpr (sizeof(T) == 4) rc = launch_bin_rows_t<T, 4>(stream, hs, a, b, grid);
@@ -1090,7 +1071,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   }
   TileWalk w;
   unsigned grid = 0;
-  LBT_TRY(fill_walk(w, hs, b, n_cu, hs.n_groups, use_cache ? hs.brpp : hs.rpp,
+  LBT_TRY(fill_walk(w, b, n_cu, hs.n_groups, use_cache ? hs.brpp : hs.rpp,
                     use_cache ? (hs.bvec == 16 ? kBinnedUnroll / 2 : kBinnedUnroll) : kUnroll,
                     use_cache ? hs.blds_bytes : hs.lds_bytes, &grid));
   {
@@ -1107,18 +1088,16 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   if (use_cache) {
     BinnedArgs a;
     a.w            = w;
-    a.bin_base     = hs.bin_base;
-    a.bin_stride   = hs.bin_stride;
+    a.rec          = hs.rec;
     a.K            = b.K;
     a.row_pointers = b.row_pointers;
     a.groups       = hs.groups;
     a.hist         = b.hist;
-    if (hs.bin_bytes == 1 && hs.bvec == 16) return launch_binned<uint8_t, 16>(stream, hs, a, b, grid);
     if (hs.bin_bytes == 1)
-      return hs.bvec == 4 ? launch_binned<uint8_t, 4>(stream, hs, a, b, grid)
-                          : launch_binned<uint8_t, 1>(stream, hs, a, b, grid);
-    return hs.bvec == 4 ? launch_binned<uint16_t, 4>(stream, hs, a, b, grid)
-                        : launch_binned<uint16_t, 1>(stream, hs, a, b, grid);
+      return hs.embed ? launch_binned<uint8_t, 16, true>(stream, hs, a, b, grid)
+                      : launch_binned<uint8_t, 16, false>(stream, hs, a, b, grid);
+    return hs.embed ? launch_binned<uint16_t, 4, true>(stream, hs, a, b, grid)
+                    : launch_binned<uint16_t, 4, false>(stream, hs, a, b, grid);
   }
   HistArgs<T> a;
   a.w            = w;
@@ -1142,7 +1121,8 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
 }
 
 // Packs consecutive features, `unit` at a time, into groups whose LDS need
-// (bytes_of(feature)) stays within the budget; a second pass balances widths.
+// (bytes_of(feature)) stays within the budget and whose rows take at most half a
+// workgroup of lanes (lane_vec features per lane); a second pass balances widths.
 template <typename BytesOf>
 size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_of, std::vector<int32_t>& groups)
 {
@@ -1172,7 +1152,7 @@ size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_o
   const int n_min = static_cast<int>(groups.size()) - 1;
   int target      = (F + n_min - 1) / n_min;
   target          = ((target + unit - 1) / unit) * unit;
-  pack(target);    // same count, balanced widths
+  pack(target);    // same count where the budget allows, balanced widths
   return lds;
 }
 
@@ -1186,9 +1166,21 @@ int rows_per_pass(const std::vector<int32_t>& groups, int vec)
   return rpp;
 }
 
+template <typename BytesOf>
+size_t widest_group(const std::vector<int32_t>& groups, BytesOf bytes_of)
+{
+  size_t need = 0;
+  for (size_t g = 0; g + 1 < groups.size(); g++) {
+    size_t sb = 0;
+    for (int f = groups[g]; f < groups[g + 1]; f++) sb += bytes_of(f);
+    need = std::max(need, sb);
+  }
+  return need;
+}
+
 }  // namespace
 
-int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t n_rows,
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, int64_t n_rows,
                  const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
                  const void* X)
 {
@@ -1205,88 +1197,108 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t 
   while ((1 << hs.search_steps) < max_feature_bins + 1) hs.search_steps++;
   const bool cached = hs.binned != nullptr;
   hs.bin_bytes      = max_feature_bins <= 256 ? 1 : 2;
-  // cached bins a lane of the histogram kernel loads at once: 16 bytes of one-byte bins
-  hs.bvec = !cached ? 1 : (hs.bin_bytes == 1 ? 16 : 4);
-  const int unit = cached ? std::max(vec, hs.bvec) : vec;
+  // cached bins a lane of the histogram kernel loads at once: 16 one-byte or 4 two-byte bins
+  hs.bvec  = !cached ? 1 : (hs.bin_bytes == 1 ? 16 : 4);
+  hs.embed = cached && K == 1;
 
-  // LDS a feature needs: the search side keeps proposals and a lookup table; the packed
-  // sub-histogram joins them unless the bins are cached (then the root pass only bins and the
-  // histogram kernel keeps nothing but the sub-histogram)
+  // LDS a feature needs. Search side: proposals and a lookup table, plus the packed
+  // sub-histogram when the same kernel accumulates (cache off). Histogram side with the
+  // cache: the packed sub-histogram only.
   auto search_bytes = [&](int f, int cells) {
-    return static_cast<size_t>(rp[f + 1] - rp[f]) * (cached ? elem : 8 + elem) + static_cast<size_t>(cells) * 2;
+    return static_cast<size_t>(rp[f + 1] - rp[f]) * (cached ? elem : 8 + elem) + static_cast<size_t>(cells) * 2 +
+           (cached ? kProbePad * elem : 0);
   };
   auto hist_bytes = [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; };
-  std::vector<int32_t> groups;
-  size_t budget = kLdsBudget;
-  size_t lds    = 0;
+
+  // search groups: as few as the LDS allows with the smallest table ...
+  std::vector<int32_t> sgroups;
+  const size_t search_budget = kLdsBudget - 64;  // room for the slack entries and alignment
+  size_t budget              = search_budget;
   for (;;) {
-    // groups as wide as the tighter of the two kernels allows, with the smallest table
-    lds = pack_groups(F, unit, cached ? std::min(vec, hs.bvec) : vec, budget - (cached ? 8 * kHistThreads : 0),
-                      [&](int f) { return std::max(search_bytes(f, 64), cached ? hist_bytes(f) : 0); },
-                      groups);
-    size_t need = 0;
-    for (size_t g = 0; g + 1 < groups.size(); g++) {
-      size_t sb = 0;
-      for (int f = groups[g]; f < groups[g + 1]; f++) sb += search_bytes(f, 64);
-      need = std::max(need, sb);
-    }
-    if (lds <= kLdsBudget && need <= kLdsBudget) break;
+    pack_groups(F, vec, vec, budget, [&](int f) { return search_bytes(f, 64); }, sgroups);
+    const size_t need = widest_group(sgroups, [&](int f) { return search_bytes(f, 64); });
+    if (need <= search_budget) break;
     if (budget <= 16 * 1024) {
-      set_error("a feature group does not fit the LDS (%zu bytes)", std::max(lds, need));
+      set_error("a feature group does not fit the LDS (%zu bytes)", need);
       return LBT_ERR_UNSUPPORTED;
     }
     budget -= 16 * 1024;
   }
-  // table size: the largest, up to four cells per proposal, that still fits these groups
+  // ... then the largest table, up to four cells per proposal, that still fits these groups
   int cells = 64;
-  size_t search_lds = 0;
-  for (int c = 64; c <= kMaxCells && c <= 4 * std::max(16, max_feature_bins); c <<= 1) {
-    size_t need = 0;
-    for (size_t g = 0; g + 1 < groups.size(); g++) {
-      size_t sb = 0;
-      for (int f = groups[g]; f < groups[g + 1]; f++) sb += search_bytes(f, c);
-      need = std::max(need, sb);
-    }
-    if (need > kLdsBudget) break;
+  size_t search_lds = widest_group(sgroups, [&](int f) { return search_bytes(f, 64); });
+  for (int c = 128; c <= kMaxCells && c <= 4 * std::max(16, max_feature_bins); c <<= 1) {
+    const size_t need = widest_group(sgroups, [&](int f) { return search_bytes(f, c); });
+    if (need > search_budget) break;
     cells      = c;
     search_lds = need;
   }
   hs.cells     = cells;
-  hs.n_groups  = static_cast<int>(groups.size()) - 1;
-  hs.lds_bytes = (search_lds + 15) & ~size_t(15);
-  hs.rpp       = rows_per_pass(groups, vec);
-  LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
-  if (cached) {
-    size_t blds = 0;
-    for (size_t g = 0; g + 1 < groups.size(); g++) {
-      size_t hb = 0;
-      for (int f = groups[g]; f < groups[g + 1]; f++) hb += hist_bytes(f);
-      blds = std::max(blds, hb);
+  hs.n_sgroups = static_cast<int>(sgroups.size()) - 1;
+  hs.lds_bytes = (search_lds + (cached ? kProbeSlack * elem : 0) + 15) & ~size_t(15);
+  hs.rpp       = rows_per_pass(sgroups, vec);
+  LBT_HIP(hipMemcpyAsync(hs.sgroups, sgroups.data(), sizeof(int32_t) * sgroups.size(), hipMemcpyHostToDevice, stream));
+
+  std::vector<int32_t> groups;
+  std::vector<int64_t> base(F);
+  std::vector<int32_t> stride(F), tail(F, 0);
+  std::vector<RecInfo> rec;
+  if (!cached) {
+    // one kernel searches and accumulates: the search groups are the histogram groups
+    groups       = sgroups;
+    hs.n_groups  = hs.n_sgroups;
+    hs.groups    = hs.sgroups;
+  } else {
+    // histogram groups hold whole lanes of the binning pass (multiples of vec features)
+    const size_t hbudget = kLdsBudget - 8 * kHistThreads;  // one spare slot per lane
+    pack_groups(F, vec, hs.bvec, hbudget, hist_bytes, groups);
+    const size_t blds = widest_group(groups, hist_bytes);
+    if (blds > hbudget) {
+      set_error("the bins of one feature group do not fit the LDS (%zu bytes)", blds);
+      return LBT_ERR_UNSUPPORTED;
     }
-    hs.blds_bytes = (blds + 8 * kHistThreads + 15) & ~size_t(15);  // + one spare slot per lane
+    hs.n_groups   = static_cast<int>(groups.size()) - 1;
+    hs.blds_bytes = (blds + 8 * kHistThreads + 15) & ~size_t(15);
     hs.brpp       = rows_per_pass(groups, hs.bvec);
-    // the cache: one array per group, [row][features of the group padded to 32 bytes]
-    std::vector<int64_t> base(F);
-    std::vector<int32_t> stride(F);
-    int64_t at = 0;
-    for (size_t g = 0; g + 1 < groups.size(); g++) {
+    LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
+    // record layout of every histogram group
+    const int chunk = hs.bvec * hs.bin_bytes;  // bytes a lane of the histogram kernel loads
+    int64_t at      = 0;
+    rec.resize(hs.n_groups);
+    for (int g = 0; g < hs.n_groups; g++) {
       const int gs        = groups[g + 1] - groups[g];
-      const int64_t pitch = (static_cast<int64_t>(gs) * hs.bin_bytes + 31) / 32 * 32 / hs.bin_bytes;
-      for (int f = groups[g]; f < groups[g + 1]; f++) {
-        base[f]   = at + (f - groups[g]);
-        stride[f] = static_cast<int32_t>(pitch);
+      const int bins_end  = gs * hs.bin_bytes;
+      const int chunk_end = (bins_end + chunk - 1) / chunk * chunk;
+      RecInfo& ri         = rec[g];
+      ri.bins_end         = bins_end;
+      if (hs.embed) {
+        ri.q_off    = (bins_end + 7) / 8 * 8;
+        ri.zero_end = ri.q_off;
+      } else {
+        ri.q_off    = -1;
+        ri.zero_end = chunk_end;
       }
-      at += n_rows * pitch;
+      const int used = std::max(chunk_end, hs.embed ? ri.q_off + 8 : 0);
+      ri.stride      = (used + 31) / 32 * 32;
+      ri.base        = at;
+      for (int f = groups[g]; f < groups[g + 1]; f++) {
+        base[f]   = at / hs.bin_bytes + (f - groups[g]);
+        stride[f] = ri.stride / hs.bin_bytes;
+      }
+      tail[groups[g + 1] - 1] = g + 1;
+      at += n_rows * ri.stride;
     }
-    if (at * hs.bin_bytes > n_rows * bin_row_bytes_max(F, hs.bin_bytes)) {
-      set_error("bin cache of %lld bytes exceeds the workspace share", static_cast<long long>(at * hs.bin_bytes));
+    if (static_cast<size_t>(at) > hs.binned_capacity) {
+      set_error("bin cache of %lld bytes exceeds the workspace share", static_cast<long long>(at));
       return LBT_ERR_WORKSPACE;
     }
+    LBT_HIP(hipMemcpyAsync(hs.rec, rec.data(), sizeof(RecInfo) * rec.size(), hipMemcpyHostToDevice, stream));
     LBT_HIP(hipMemcpyAsync(hs.bin_base, base.data(), sizeof(int64_t) * F, hipMemcpyHostToDevice, stream));
     LBT_HIP(hipMemcpyAsync(hs.bin_stride, stride.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
-    // the host vectors must outlive the asynchronous copies
-    LBT_HIP(hipStreamSynchronize(stream));
+    LBT_HIP(hipMemcpyAsync(hs.bin_tail, tail.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
   }
+  // the host vectors must outlive the asynchronous copies
+  LBT_HIP(hipStreamSynchronize(stream));
   ProfScope ps(LBT_PROF_PROPOSALS, stream);
   if (is_f64)
     build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,

@@ -255,48 +255,70 @@ struct LevelMeta {
 };
 
 
-// Per-tree state of the histogram stage: feature groups sized for the LDS of
-// one workgroup and, per feature, a table that maps a value to the first
-// split proposal it can reach (see lbt_histogram.hip).
+// Where the records of one histogram feature group live in the bin cache. A record is what
+// one row contributes to the group: the feature-relative bins of the group's features, zero
+// bytes up to zero_end, and (single-output trees) the row's packed (grad, hess) pair at q_off.
+struct RecInfo {
+  int64_t base;      // byte offset of row 0's record
+  int32_t stride;    // bytes between consecutive rows (multiple of 32)
+  int32_t q_off;     // byte offset of the int2 (grad, hess) inside a record, or -1
+  int32_t zero_end;  // bytes [bins_end, zero_end) of a record are zero
+  int32_t bins_end;  // bytes of bins in a record
+};
+
+// Per-tree state of the histogram stage (see lbt_histogram.hip).
 struct HistSetup {
   int n_features     = 0;
-  int n_groups       = 0;
-  int vec            = 1;   // features per lane (1, 2 or 4)
+  int n_groups       = 0;   // histogram feature groups (LDS holds a group's packed sub-histogram)
+  int n_sgroups      = 0;   // search feature groups (LDS holds proposals and lookup tables)
+  int vec            = 1;   // features per lane of the search (1, 2 or 4)
   int cells          = 0;   // table entries per feature (power of two)
   int search_steps   = 0;   // ceil(log2(max bins of a feature + 1))
-  size_t lds_bytes   = 0;
+  size_t lds_bytes   = 0;   // LDS of the search / binning kernel
   bool is_f64        = false;
   // device buffers (carved from the caller's workspace)
   int32_t* groups    = nullptr;  // [n_groups + 1]
+  int32_t* sgroups   = nullptr;  // [n_sgroups + 1]; the same array as groups when the cache is off
   uint16_t* tables   = nullptr;  // [n_features][cells]
   void* cell_lo      = nullptr;  // X dtype [n_features]
   void* cell_invw    = nullptr;  // X dtype [n_features]
   int32_t* tile_start = nullptr;
   int4* tiles         = nullptr;  // one descriptor per tile of the batch in flight
   LevelMeta* meta    = nullptr;
-  // bin cache: feature-relative bin of every (row, feature), written by the root binning
-  // pass and read by the histogram kernel of every level instead of X. When it is in use the
-  // groups above serve both kernels and the cache is stored group by group:
-  // [group][row][features of the group, padded to a 32-byte sector].
-  void* binned         = nullptr;  // uint8 or uint16, or null (cache off)
+  // bin cache: written by the root binning pass and read by the histogram kernel of every
+  // level instead of X; stored histogram group by histogram group as [group][row][record]
+  void* binned         = nullptr;  // null: cache off
+  size_t binned_capacity = 0;      // bytes available at `binned`
   int bin_bytes        = 0;        // 1 or 2
   int bvec             = 1;        // cached bins a lane of the histogram kernel loads at once
+  bool embed           = false;    // records carry the row's (grad, hess)
   size_t blds_bytes    = 0;        // LDS of the histogram kernel (packed sub-histogram only)
+  RecInfo* rec         = nullptr;  // [n_groups]
   int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
   int32_t* bin_stride  = nullptr;  // [n_features] elements between consecutive rows
+  int32_t* bin_tail    = nullptr;  // [n_features] g + 1 for the last feature of histogram group g, else 0
   int rpp              = 0;        // rows per workgroup pass, search / binning kernel
   int brpp             = 0;        // rows per workgroup pass, histogram kernel on cached bins
 };
 
 constexpr int kMaxCells = 2048;
 constexpr int kTransposeFeatures = 64;  // features the bin transpose stages at a time
+constexpr int kHistThreads       = 1024;
+// LDS a histogram-stage workgroup may fill; 4 KB of the 160 KB stay free for the tile window
+constexpr size_t kLdsBudget = 160 * 1024 - 512 - 4096;
 
-// Upper bound on the bytes of one row of the bin cache (features plus sector padding
-// between groups); the workspace reserves n_rows times this.
-inline int64_t bin_row_bytes_max(int n_features, int bin_bytes)
+// Upper bound on the cache bytes one row can take for n_features features with at most
+// split_samples bins each: the bins plus, per histogram group, the embedded gradient pair,
+// alignment and padding to the 32-byte record pitch. The group count is bounded through the
+// fewest features a group can hold.
+inline int64_t bin_row_bytes_max(int n_features, int split_samples)
 {
-  int64_t raw = static_cast<int64_t>(n_features) * bin_bytes;
-  return (raw + raw / 4 + 31) / 32 * 32 + 64;
+  const int bin_bytes = split_samples <= 256 ? 1 : 2;
+  int64_t cap = static_cast<int64_t>((kLdsBudget - 8 * kHistThreads) / (8 * static_cast<size_t>(split_samples)));
+  if (cap >= 4) cap = cap / 4 * 4;
+  if (cap < 1) cap = 1;
+  const int64_t groups_max = (n_features + cap - 1) / cap + 1;
+  return static_cast<int64_t>(n_features) * bin_bytes + groups_max * 48;
 }
 
 struct HistBatch {
@@ -311,6 +333,7 @@ struct HistBatch {
   int level_first;
   const void* proposals;
   const int32_t* row_pointers;
+  const int32_t* bin_feature;  // [bins] feature of every proposal
   HistView hist;
   const unsigned long long* qstats;
   const I64Pair* node_sums;
@@ -320,7 +343,7 @@ struct HistBatch {
 
 // Chooses groups / table size from the host copy of the row pointers and builds
 // the tables on the device.
-int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int64_t n_rows,
+int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, int64_t n_rows,
                  const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
                  const void* X);
 // Plans tiles for the batch and launches the histogram kernel.
