@@ -6,7 +6,7 @@ Tree(max_depth=8, split_samples=256), X 10,000,000 x 100 f32. One step is one
 boosting round: gradient step, BuildTreeTask, PredictTask of the new tree and
 the prediction update, all with inputs resident in HBM.
 
-Prints ONE JSON line. `roofline` describes the histogram kernel (HIP events on
+Prints ONE JSON line. `roofline` describes the histogram kernels (HIP events on
 the stream of the call, summed over the timed rounds); `cpu_baseline` is the
 restated CPU variant of the reference timed on the host cores of this machine
 on a row sample of the same workload.
@@ -86,6 +86,25 @@ def cpu_baseline_build(X_sample, y_sample, max_depth, split_samples, lr, full_ro
     }
 
 
+def measured_traffic(workload, rows, features):
+    """HBM bytes per launch from rocprofv3 counter runs of this command, kept as text under profiles/.
+
+    Lines of the form `<kernel> traffic_bytes_per_launch=<number> workload=<name> rows=<n> features=<f>`;
+    only those taken on the same workload apply. Returns {} when none do."""
+    out = {}
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_%s.txt" % workload)
+    if not os.path.exists(path):
+        return out
+    for line in open(path):
+        parts = line.split()
+        if len(parts) < 2 or "traffic_bytes_per_launch=" not in line:
+            continue
+        kv = dict(p.split("=", 1) for p in parts[1:] if "=" in p)
+        if kv.get("workload") == workload and int(kv.get("rows", -1)) == rows and int(kv.get("features", -1)) == features:
+            out[parts[0]] = float(kv["traffic_bytes_per_launch"])
+    return out
+
+
 def bench_training(args):
     import numpy as np
     import torch
@@ -163,13 +182,33 @@ def bench_training(args):
     prof = _lib.profile_get()
     loss1 = loss()
 
-    hist = prof["histogram"]
-    achieved = hist["bytes"] / (hist["ms"] * 1e-3) / 1e9 if hist["ms"] > 0 else 0.0
-    levels = [
-        {"level": d, "ms": lv["ms"] / args.steps, "GB": lv["bytes"] / args.steps / 1e9,
-         "GBps": (lv["bytes"] / (lv["ms"] * 1e-3) / 1e9) if lv["ms"] > 0 else 0.0}
-        for d, lv in enumerate(prof["levels"])
-    ]
+    hist, binning = prof["histogram"], prof["binning"]
+    elem = X.element_size()
+    bin_bytes = 1 if S <= 256 else 2
+    steps = args.steps
+
+    def gbps(byts, ms):
+        return byts / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+
+    # Algorithmic bytes of the histogram stage per level, the reference kernel's accounting:
+    # every row of a built node reads its F feature values of X and its packed (grad, hess)
+    # per output (gradients are quantised once per tree, 8 bytes per pair), every row of the
+    # level's nodes its (node, row) pair, every built histogram is written once.
+    stage_bytes = 0.0
+    levels = []
+    for d, lv in enumerate(prof["levels"]):
+        # the library's own figure prices a feature value at its cached width; what is left of it
+        # after the row terms are the histograms written
+        written = max(0.0, lv["bytes"] - lv["built_instances"] * (f * bin_bytes + k * 8.0 + 8.0))
+        ref_bytes = lv["built_instances"] * (f * elem + k * 8.0) + lv["instances"] * 8.0 + written
+        stage_bytes += ref_bytes
+        levels.append({"level": d, "ms": lv["ms"] / steps, "built_rows": lv["built_instances"] / steps,
+                       "built_nodes": lv["built_nodes"] / steps,
+                       "GB_cached_bins": lv["bytes"] / steps / 1e9, "GBps_cached_bins": gbps(lv["bytes"], lv["ms"]),
+                       "GB_reference_accounting": ref_bytes / steps / 1e9})
+    stage_ms = hist["ms"] + binning["ms"]
+    traffic = measured_traffic(name, n, f)
+    hist_achieved = gbps(hist["bytes"], hist["ms"])
     out = {
         "metric": "boosting rounds/sec + histogram HBM GB/s (% peak), 10M×100 depth 8" if cfg == 2
         else "boosting rounds/sec + histogram HBM GB/s (%% peak), %s" % name,
@@ -192,23 +231,38 @@ def bench_training(args):
             "loss_before": loss0, "loss_after": loss1,
             "prediction_update": "PredictTask" if args.reference_flow else "row->leaf map from BuildTreeTask",
         },
+        # the kernel with the largest share of a round: the histogram kernel on cached bins,
+        # priced on the bytes of its own input format (one or two bytes per feature value)
         "roofline": {
             "bound": "hbm",
-            "achieved": achieved,
+            "achieved": hist_achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
-            "kernel": "histogram_kernel",
+            "frac": hist_achieved / HBM_PEAK_GBS,
+            "traffic": traffic.get("binned_histogram_kernel"),
+            "kernel": "binned_histogram_kernel",
             "launches": hist["launches"],
             "avg_launch_ms": hist["ms"] / max(1, hist["launches"]),
-            "bytes_per_round": hist["bytes"] / args.steps,
+            "bytes_per_launch": hist["bytes"] / max(1, hist["launches"]),
             "levels": levels,
+            # the other kernel of the histogram stage: the root pass that bins X into the cache
+            "binning_kernel": {
+                "kernel": "bin_rows_kernel", "launches": binning["launches"],
+                "avg_launch_ms": binning["ms"] / max(1, binning["launches"]),
+                "bytes_per_launch": binning["bytes"] / max(1, binning["launches"]),
+                "achieved": gbps(binning["bytes"], binning["ms"]),
+                "frac": gbps(binning["bytes"], binning["ms"]) / HBM_PEAK_GBS,
+                "traffic": traffic.get("bin_rows_kernel"),
+            },
+            # the whole histogram stage of a tree (both kernels) against the bytes the
+            # reference's histogram kernel would have to move for the same levels
+            "stage_reference_accounting": {
+                "kernels": "bin_rows_kernel + binned_histogram_kernel",
+                "ms_per_tree": stage_ms / steps, "GB_per_tree": stage_bytes / steps / 1e9,
+                "achieved": gbps(stage_bytes, stage_ms), "frac": gbps(stage_bytes, stage_ms) / HBM_PEAK_GBS,
+            },
         },
         "kernel_ms_per_round": {c: prof[c]["ms"] / args.steps for c in _lib.PROF_CLASSES},
-        "binning": {"ms": prof["binning"]["ms"] / args.steps, "GB": prof["binning"]["bytes"] / args.steps / 1e9,
-                    "GBps": (prof["binning"]["bytes"] / (prof["binning"]["ms"] * 1e-3) / 1e9)
-                    if prof["binning"]["ms"] > 0 else 0.0},
     }
     if not args.no_cpu_baseline:
         ns = min(n, 500_000 if cfg != 1 else n)

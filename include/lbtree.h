@@ -159,6 +159,11 @@ typedef struct lbt_profile {
   int32_t n_levels;
   double level_ms[64];
   double level_bytes[64];
+  /* what those launches processed: rows of all nodes of the level, rows of the nodes whose
+   * histogram was built, and the number of built nodes */
+  double level_instances[64];
+  double level_built_instances[64];
+  double level_built_nodes[64];
 } lbt_profile;
 
 /* When enabled, lbt_build_tree / lbt_predict bracket their kernels with HIP

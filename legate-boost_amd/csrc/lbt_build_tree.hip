@@ -1301,6 +1301,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * per_value + K * 8.0 + 8.0) +
                   static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
       acc.level_bytes[d] += by;
+      acc.level_instances[d] += static_cast<double>(h_levels[d].instances);
+      acc.level_built_instances[d] += static_cast<double>(h_levels[d].built_instances);
+      acc.level_built_nodes[d] += static_cast<double>(h_levels[d].built_nodes);
       acc.bytes[LBT_PROF_HISTOGRAM] += by;
     }
   }

@@ -1034,8 +1034,11 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
   if (use_cache && depth == 0) {
     // fill the bin cache: rows split evenly over as many workgroups as are resident at once
+    // X read once, one bin written per value; with embedded gradients also one pair read and
+    // one written per row and histogram group
     ProfScope ps(LBT_PROF_BINNING, stream,
-                 static_cast<double>(b.n_rows) * b.F * (sizeof(T) + static_cast<double>(hs.bin_bytes)));
+                 static_cast<double>(b.n_rows) * b.F * (sizeof(T) + static_cast<double>(hs.bin_bytes)) +
+                   (hs.embed ? static_cast<double>(b.n_rows) * 8.0 * (1 + hs.n_groups) : 0.0));
     BinRowsArgs<T> a;
     a.F            = b.F;
     a.n_rows       = b.n_rows;

@@ -60,6 +60,9 @@ class Profile(C.Structure):
         ("n_levels", C.c_int32),
         ("level_ms", C.c_double * 64),
         ("level_bytes", C.c_double * 64),
+        ("level_instances", C.c_double * 64),
+        ("level_built_instances", C.c_double * 64),
+        ("level_built_nodes", C.c_double * 64),
     ]
 
 
@@ -128,5 +131,7 @@ def profile_get():
     out = {}
     for i, name in enumerate(PROF_CLASSES):
         out[name] = {"launches": p.launches[i], "ms": p.ms[i], "bytes": p.bytes[i]}
-    out["levels"] = [{"ms": p.level_ms[d], "bytes": p.level_bytes[d]} for d in range(p.n_levels)]
+    out["levels"] = [{"ms": p.level_ms[d], "bytes": p.level_bytes[d], "instances": p.level_instances[d],
+                      "built_instances": p.level_built_instances[d], "built_nodes": p.level_built_nodes[d]}
+                     for d in range(p.n_levels)]
     return out
