@@ -1,0 +1,179 @@
+// Legate-side binding of liblbtree.so: the bodies a maintainer of
+// rapidsai/legate-boost drops in for the GPU variants of the three tree tasks
+// when building for MI355X. Task classes, op codes, registration and the Python
+// layer stay as they are (src/models/tree/build_tree.h:308-317,
+// src/legate_library.h:23-33, legateboost/models/tree.py:104-280).
+//
+// This file needs the Legate headers and is therefore not compiled by this
+// repository's build; it documents, in code, which task argument lands in which
+// parameter of the C ABI.
+//
+//   BuildTreeTask::gpu_variant  replaces src/models/tree/build_tree.cu:1274-1365
+//   PredictTask::gpu_variant    replaces src/models/tree/predict.cu:26-91
+//   UpdateTreeTask::gpu_variant is new (the reference has a CPU variant only,
+//                               src/models/tree/update_tree.cc:36-133)
+#include <legate.h>
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "lbtree.h"
+#include "models/tree/build_tree.h"
+#include "models/tree/predict.h"
+#include "models/tree/update_tree.h"
+
+namespace legateboost {
+namespace {
+
+void check(int status)
+{
+  if (status != LBT_OK) throw std::runtime_error(std::string("lbtree: ") + lbt_last_error());
+}
+
+int x_dtype(const legate::PhysicalStore& X)
+{
+  if (X.code() == legate::Type::Code::FLOAT32) return LBT_F32;
+  if (X.code() == legate::Type::Code::FLOAT64) return LBT_F64;
+  throw std::runtime_error("lbtree: X must be float32 or float64");
+}
+
+// Dense, C-ordered instances only (the mapper requests exactly that for these tasks,
+// src/mapper.cc:49-58): the pointer of the first element is then all the library needs.
+template <typename T, int DIM>
+const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
+{
+  *shape = s.shape<DIM>();
+  if (shape->empty()) return nullptr;
+  size_t strides[DIM];
+  const T* p = s.read_accessor<T, DIM>().ptr(*shape, strides);
+  return p;
+}
+
+}  // namespace
+
+/*static*/ void BuildTreeTask::gpu_variant(legate::TaskContext context)
+{
+  const auto X_store = context.input(0).data();
+  legate::Rect<3> xs, gs, hs;
+  const int dtype    = x_dtype(X_store);
+  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
+                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
+  const double* g    = dense_in<double, 3>(context.input(1).data(), &gs);
+  const double* h    = dense_in<double, 3>(context.input(2).data(), &hs);
+  const int64_t rows = std::max<int64_t>(xs.hi[0] - xs.lo[0] + 1, 0);
+  const int features = static_cast<int>(xs.hi[1] - xs.lo[1] + 1);
+  const int outputs  = static_cast<int>(gs.hi[2] - gs.lo[2] + 1);
+
+  lbt_build_params p{};
+  p.max_depth         = context.scalars().at(0).value<int>();
+  p.max_nodes         = context.scalars().at(1).value<int>();
+  p.split_samples     = context.scalars().at(2).value<int>();
+  p.seed              = context.scalars().at(3).value<int>();
+  p.dataset_rows      = context.scalars().at(4).value<int64_t>();
+  p.l1_regularization = context.scalars().at(5).value<double>();
+  p.l2_regularization = context.scalars().at(6).value<double>();
+  p.min_split_gain    = context.scalars().at(7).value<double>();
+  p.hist_cache_bytes  = 0;  // the reference's 1e9-byte histogram budget
+
+  const uint8_t* feature_set = nullptr;
+  if (context.inputs().size() == 4) {
+    legate::Rect<1> fs;
+    feature_set = reinterpret_cast<const uint8_t*>(dense_in<bool, 1>(context.input(3).data(), &fs));
+  }
+
+  // outputs 0..4: leaf, feature, split, gain, hessian (build_tree.cu:830-842)
+  auto out_ptr = [&](int i, auto tag, auto dim) {
+    using T          = decltype(tag);
+    constexpr int D  = decltype(dim)::value;
+    auto store       = context.output(i).data();
+    auto shape       = store.template shape<D>();
+    size_t strides[D];
+    return store.template write_accessor<T, D>().ptr(shape, strides);
+  };
+  double* leaf     = out_ptr(0, double{}, std::integral_constant<int, 2>{});
+  int32_t* feature = out_ptr(1, int32_t{}, std::integral_constant<int, 1>{});
+  double* split    = out_ptr(2, double{}, std::integral_constant<int, 1>{});
+  double* gain     = out_ptr(3, double{}, std::integral_constant<int, 1>{});
+  double* hessian  = out_ptr(4, double{}, std::integral_constant<int, 2>{});
+
+  // task-scoped scratch from Legate's pool, as the reference takes its buffers
+  // (build_tree.cu:790-794, :880-933, :997); the task already declares allocations
+  const size_t ws_bytes =
+    lbt_build_tree_workspace_bytes(rows, features, outputs, p.max_depth, p.split_samples, dtype, p.hist_cache_bytes);
+  auto workspace = legate::create_buffer<int8_t>(ws_bytes, legate::Memory::GPU_FB_MEM, 256);
+
+  // With more than one GPU the four exchanges of the reference (scale, proposals, root sums,
+  // histogram batches: build_tree.cu:89-93, :901-902, :1170-1174, :1107-1113) would be made
+  // here between library stages; this binding is the single-GPU task.
+  check(lbt_build_tree(context.get_task_stream(), X, dtype, xs.lo[0], rows, features, g, h, outputs, feature_set, &p,
+                       leaf, feature, split, gain, hessian, workspace.ptr(0), ws_bytes, nullptr));
+  workspace.destroy();
+}
+
+/*static*/ void PredictTask::gpu_variant(legate::TaskContext context)
+{
+  const auto X_store = context.input(0).data();
+  legate::Rect<3> xs;
+  const int dtype    = x_dtype(X_store);
+  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
+                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
+  const int64_t rows = xs.hi[0] - xs.lo[0] + 1;
+  if (rows < 1) return;
+  auto pred          = context.output(0).data();
+  auto pred_shape    = pred.shape<3>();
+  size_t strides[3];
+  double* out       = pred.write_accessor<double, 3>().ptr(pred_shape, strides);
+  const int outputs = static_cast<int>(pred_shape.hi[2] - pred_shape.lo[2] + 1);
+
+  // inputs 1.. are (leaf, feature, split) per tree (legateboost/models/tree.py:264-273)
+  std::vector<const double*> leaf, split;
+  std::vector<const int32_t*> feature;
+  std::vector<int32_t> nodes;
+  for (size_t i = 1; i + 2 < context.inputs().size(); i += 3) {
+    legate::Rect<2> ls;
+    legate::Rect<1> fs, ss;
+    leaf.push_back(dense_in<double, 2>(context.input(i).data(), &ls));
+    feature.push_back(dense_in<int32_t, 1>(context.input(i + 1).data(), &fs));
+    split.push_back(dense_in<double, 1>(context.input(i + 2).data(), &ss));
+    nodes.push_back(static_cast<int32_t>(fs.hi[0] - fs.lo[0] + 1));
+  }
+  check(lbt_predict(context.get_task_stream(), X, dtype, rows, static_cast<int>(xs.hi[1] - xs.lo[1] + 1),
+                    static_cast<int>(leaf.size()), leaf.data(), feature.data(), split.data(), nodes.data(), outputs,
+                    out));
+}
+
+/*static*/ void UpdateTreeTask::gpu_variant(legate::TaskContext context)
+{
+  const auto X_store = context.input(0).data();
+  legate::Rect<3> xs, gs, hs;
+  legate::Rect<1> fs, ss;
+  const int dtype        = x_dtype(X_store);
+  const void* X          = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
+                                            : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
+  const double* g        = dense_in<double, 3>(context.input(1).data(), &gs);
+  const double* h        = dense_in<double, 3>(context.input(2).data(), &hs);
+  const int32_t* feature = dense_in<int32_t, 1>(context.input(3).data(), &fs);
+  const double* split    = dense_in<double, 1>(context.input(4).data(), &ss);
+  const int64_t rows     = std::max<int64_t>(xs.hi[0] - xs.lo[0] + 1, 0);
+  const int outputs      = static_cast<int>(gs.hi[2] - gs.lo[2] + 1);
+  const int nodes        = static_cast<int>(fs.hi[0] - fs.lo[0] + 1);
+  const double l1        = context.scalars().at(0).value<double>();
+  const double l2        = context.scalars().at(1).value<double>();
+
+  auto leaf_store = context.output(0).data();
+  auto hess_store = context.output(1).data();
+  size_t strides[2];
+  double* leaf    = leaf_store.write_accessor<double, 2>().ptr(leaf_store.shape<2>(), strides);
+  double* hessian = hess_store.write_accessor<double, 2>().ptr(hess_store.shape<2>(), strides);
+
+  const size_t ws_bytes = lbt_update_tree_workspace_bytes(rows, outputs, nodes);
+  auto workspace        = legate::create_buffer<int8_t>(ws_bytes, legate::Memory::GPU_FB_MEM, 256);
+  // more than one GPU: all-reduce the per-node sums before the leaves are recomputed, where the
+  // reference's CPU variant calls SumAllReduce (update_tree.cc:96-104)
+  check(lbt_update_tree(context.get_task_stream(), X, dtype, rows, static_cast<int>(xs.hi[1] - xs.lo[1] + 1), g, h,
+                        outputs, feature, split, nodes, l1, l2, leaf, hessian, workspace.ptr(0), ws_bytes));
+  workspace.destroy();
+}
+
+}  // namespace legateboost
