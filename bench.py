@@ -171,16 +171,24 @@ def bench_training(args):
     for _ in range(args.warmup):
         one_round()
     torch.cuda.synchronize()
+    # the timed rounds carry HIP events around the two histogram-stage kernels only (18 events
+    # per round); the per-class breakdown comes from two further, untimed rounds
     _lib.profile_reset()
-    _lib.profile_enable(True)
+    _lib.profile_enable(2)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         one_round()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    _lib.profile_enable(False)
     prof = _lib.profile_get()
     loss1 = loss()
+    _lib.profile_reset()
+    _lib.profile_enable(1)
+    for _ in range(2):
+        one_round()
+    torch.cuda.synchronize()
+    _lib.profile_enable(0)
+    prof_all = _lib.profile_get()
 
     hist, binning = prof["histogram"], prof["binning"]
     elem = X.element_size()
@@ -262,7 +270,8 @@ def bench_training(args):
                 "achieved": gbps(stage_bytes, stage_ms), "frac": gbps(stage_bytes, stage_ms) / HBM_PEAK_GBS,
             },
         },
-        "kernel_ms_per_round": {c: prof[c]["ms"] / args.steps for c in _lib.PROF_CLASSES},
+        # two rounds after the timed ones, every kernel class bracketed by events
+        "kernel_ms_per_round": {c: prof_all[c]["ms"] / 2 for c in _lib.PROF_CLASSES},
     }
     if not args.no_cpu_baseline:
         ns = min(n, 500_000 if cfg != 1 else n)

@@ -1254,7 +1254,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
 
   // ---- observation points
   std::vector<LevelMeta> h_levels(max_depth > 0 ? max_depth : 1);
-  const bool want_levels = max_depth > 0 && (profiler().enabled || (taps && (taps->level_instances || taps->level_built_instances || taps->level_built_nodes)));
+  const bool want_levels = max_depth > 0 && ((profiler().mode != 0) || (taps && (taps->level_instances || taps->level_built_instances || taps->level_built_nodes)));
   if (want_levels)
     LBT_HIP(hipMemcpyAsync(h_levels.data(), L.level_totals, sizeof(LevelMeta) * max_depth, hipMemcpyDeviceToHost, stream));
   if (taps) {
@@ -1288,7 +1288,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       if (taps && taps->level_built_nodes) taps->level_built_nodes[d] = static_cast<int32_t>(h_levels[d].built_nodes);
     }
   }
-  if (profiler().enabled) {
+  if ((profiler().mode != 0)) {
     profiler().collect();
     // algorithmic bytes of the histogram launches of each level:
     // X rows of built nodes + their packed gradients + one position pair per
@@ -1367,7 +1367,7 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
   else
     rc = lbt::build_tree_impl<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, g, h,
                                       n_outputs, feature_set, *params, leaf, feature, split, gain, hessian, L, taps);
-  if (rc != LBT_OK && lbt::profiler().enabled) {
+  if (rc != LBT_OK && lbt::profiler().mode != 0) {
     (void)hipStreamSynchronize(s);
     lbt::profiler().collect();
   }

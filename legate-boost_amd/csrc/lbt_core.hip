@@ -27,7 +27,20 @@ void Profiler::begin(int cls, int level, double bytes, hipStream_t s)
   sp.cls   = cls;
   sp.level = level;
   sp.bytes = bytes;
-  if (hipEventCreate(&sp.start) != hipSuccess || hipEventCreate(&sp.stop) != hipSuccess) return;
+  // events are kept and reused: creating a pair per span costs more than recording it
+  auto take = [&](hipEvent_t* e) {
+    if (!pool.empty()) {
+      *e = pool.back();
+      pool.pop_back();
+      return true;
+    }
+    return hipEventCreate(e) == hipSuccess;
+  };
+  if (!take(&sp.start)) return;
+  if (!take(&sp.stop)) {
+    pool.push_back(sp.start);
+    return;
+  }
   (void)hipEventRecord(sp.start, s);
   open.push_back(sp);
 }
@@ -53,8 +66,8 @@ void Profiler::collect()
         acc.level_bytes[sp.level] += sp.bytes;
       }
     }
-    (void)hipEventDestroy(sp.start);
-    (void)hipEventDestroy(sp.stop);
+    pool.push_back(sp.start);
+    pool.push_back(sp.stop);
   }
   open.clear();
 }
@@ -67,7 +80,7 @@ const char* lbt_last_error(void) { return lbt::g_error; }
 
 int lbt_version(void) { return 1; }
 
-void lbt_profile_enable(int on) { lbt::profiler().enabled = on != 0; }
+void lbt_profile_enable(int on) { lbt::profiler().mode = on < 0 ? 0 : on; }
 
 void lbt_profile_reset(void)
 {

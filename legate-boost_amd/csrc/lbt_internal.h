@@ -77,9 +77,14 @@ struct ProfSpan {
 };
 
 struct Profiler {
-  bool enabled = false;
+  int mode = 0;  // 0 off, 1 every kernel class, 2 the two histogram-stage classes only
   lbt_profile acc{};
   std::vector<ProfSpan> open;  // spans of the call in flight
+  std::vector<hipEvent_t> pool;  // events waiting to be reused
+  bool wants(int cls) const
+  {
+    return mode == 1 || (mode == 2 && (cls == LBT_PROF_HISTOGRAM || cls == LBT_PROF_BINNING));
+  }
   void begin(int cls, int level, double bytes, hipStream_t s);
   void end(hipStream_t s);
   void collect();  // after the stream has been synchronised
@@ -91,7 +96,7 @@ struct ProfScope {
   bool on;
   ProfScope(int cls, hipStream_t stream, double bytes = 0.0, int level = -1) : s(stream)
   {
-    on = profiler().enabled;
+    on = profiler().wants(cls);
     if (on) profiler().begin(cls, level, bytes, s);
   }
   ~ProfScope()

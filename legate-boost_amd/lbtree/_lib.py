@@ -118,7 +118,8 @@ def check(rc):
 
 
 def profile_enable(on=True):
-    lib.lbt_profile_enable(1 if on else 0)
+    """True / 1: every kernel class; 2: the histogram-stage classes only; False / 0: off."""
+    lib.lbt_profile_enable(int(on))
 
 
 def profile_reset():
