@@ -108,18 +108,28 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
                    double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
                    void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
 
+/* Device scratch for lbt_predict: room for the ensemble packed into one node array
+ * (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
+size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t x_dtype);
+
 /*
  * PredictTask::gpu_variant (src/models/tree/predict.cu:26-91).
  *   leaf/feature/split  HOST arrays of n_trees device pointers, in the order
  *                       the trees appear as task inputs (tree.py:264-273)
  *   tree_nodes          HOST array: number of nodes of each tree
  *   out                 device double [n_rows][n_outputs]; overwritten
+ *   workspace           device scratch of at least lbt_predict_workspace_bytes(...), or
+ *                       NULL. With it, rows are staged in LDS in tiles of 256 and walked
+ *                       through the packed ensemble batch by batch; without it (or when a
+ *                       row tile or a tree does not fit the LDS, or n_outputs > 8) every
+ *                       node step reads the trees' own arrays. The sums are the same: a
+ *                       row's leaf values are added in tree order either way.
  * Work is enqueued on `stream`; the call does not synchronise.
  */
 int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
                 int32_t n_trees, const double* const* leaf, const int32_t* const* feature,
                 const double* const* split, const int32_t* tree_nodes, int32_t n_outputs,
-                double* out);
+                double* out, void* workspace, size_t workspace_bytes);
 
 /* Device scratch needed by lbt_update_tree. */
 size_t lbt_update_tree_workspace_bytes(int64_t n_rows, int32_t n_outputs, int32_t n_nodes);

@@ -6,6 +6,7 @@
 #include "lbt_internal.h"
 
 #include <algorithm>
+#include <vector>
 
 namespace lbt {
 namespace {
@@ -92,6 +93,400 @@ int predict_impl(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   return LBT_OK;
 }
 
+// ---- tiled traversal -------------------------------------------------------
+//
+// The ensemble is first packed into one array of nodes in the caller's workspace: threshold in
+// X's type, feature, and the index of the right child. A leaf is packed as a node that always
+// steps to itself (threshold NaN, "right child" = itself), so a walk is a fixed number of
+// identical steps with no test for leaves.
+// A workgroup then owns a tile of 256 rows: it stages the rows in LDS once and walks them
+// through all trees, a batch of up to 20 trees at a time that is copied into LDS too, so a node
+// step costs two LDS reads and no trip to the L2. Four lanes share a row and take every fourth
+// tree of the batch, five trees each, interleaved for latency. The nodes of the next batch are
+// fetched into registers while the current one is walked, and the leaf values of a batch are
+// fetched while the next one is walked. They are added in tree order, so a row's sum is formed
+// exactly as the per-tree launches of the reference form it.
+
+template <typename T>
+struct PackedNode;
+template <>
+struct alignas(8) PackedNode<float> {
+  float thr;
+  uint32_t feat_right;  // feature in the low half, right child in the high half
+};
+template <>
+struct alignas(16) PackedNode<double> {
+  double thr;
+  int32_t feat;
+  int32_t right;
+};
+
+struct alignas(16) PackedTree {
+  const double* leaf;
+  int32_t rel_off;  // first node, counted from the first node of the tree's batch
+  int32_t n_nodes;
+};
+
+struct alignas(8) BatchInfo {
+  int64_t node_off;  // first node of the batch in the packed array
+  int32_t first;     // first tree
+  int32_t count;     // trees
+  int32_t total;     // nodes
+  int32_t steps;     // steps that reach the deepest possible leaf of any tree of the batch
+};
+
+constexpr int kPackTrees    = 64;  // trees packed per launch (descriptors passed by value)
+constexpr int kPackBatches  = 128; // batch descriptors written per launch
+constexpr int kTileThreads  = 1024;
+constexpr int kTileRows     = 256;
+constexpr int kRowLanes     = 4;
+constexpr int kLaneTrees    = 5;
+constexpr int kBatchTrees   = kRowLanes * kLaneTrees;
+constexpr int kTileMaxK     = 8;
+constexpr size_t kTileLds   = 160 * 1024 - 2048;  // dynamic LDS of the tile kernel
+constexpr int kCopyWords    = 6;  // 16-byte words a thread moves per batch: 6 * 1024 * 16 B >= any batch
+constexpr int kMaxPackedNodes = 65535;  // the right child of a float node has 16 bits
+
+struct PackBatch {
+  TreeRef t[kPackTrees];
+  int64_t node_off[kPackTrees];
+  int32_t rel_off[kPackTrees];
+};
+struct BatchTable {
+  BatchInfo b[kPackBatches];
+};
+
+// x <= t for a float x holds exactly when x <= (the largest float that is <= t)
+__device__ inline float round_down_to_float(double d)
+{
+  float f = static_cast<float>(d);
+  if (static_cast<double>(f) > d) {  // false for NaN
+    uint32_t b = __float_as_uint(f);
+    if (f > 0.0f)
+      b -= 1;
+    else if (f == 0.0f)
+      b = 0x80000001u;
+    else
+      b += 1;
+    f = __uint_as_float(b);
+  }
+  return f;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+  pack_trees_kernel(PackBatch b, int first_tree, int F, PackedTree* desc, PackedNode<T>* nodes)
+{
+  const TreeRef tr = b.t[blockIdx.y];
+  const int i      = blockIdx.x * 256 + threadIdx.x;
+  if (i == 0) {
+    PackedTree d;
+    d.leaf                        = tr.leaf;
+    d.rel_off                     = b.rel_off[blockIdx.y];
+    d.n_nodes                     = tr.n_nodes;
+    desc[first_tree + blockIdx.y] = d;
+  }
+  if (i >= tr.n_nodes) return;
+  int ft = tr.feature[i];
+  // a node whose children would lie past the arrays, or whose feature does not exist, ends the walk
+  const bool is_leaf = ft < 0 || ft >= F || 2 * static_cast<int64_t>(i) + 2 >= tr.n_nodes;
+  PackedNode<T> nd;
+  // a step goes to right - (x <= thr): the comparison is false against NaN, so a leaf stays
+  const int right = is_leaf ? i : 2 * i + 2;
+  if constexpr (sizeof(T) == 4) {
+    nd.thr        = is_leaf ? __uint_as_float(0x7fc00000u) : round_down_to_float(tr.split[i]);
+    nd.feat_right = (is_leaf ? 0u : static_cast<uint32_t>(ft)) | (static_cast<uint32_t>(right) << 16);
+  } else {
+    nd.thr   = is_leaf ? __longlong_as_double(0x7ff8000000000000LL) : tr.split[i];
+    nd.feat  = is_leaf ? 0 : ft;
+    nd.right = right;
+  }
+  nodes[b.node_off[blockIdx.y] + i] = nd;
+}
+
+__global__ void write_batches_kernel(BatchTable t, int first, int n, BatchInfo* out)
+{
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[first + i] = t.b[i];
+}
+
+template <int kLane>
+__device__ inline int quad_broadcast(int v)
+{
+  // every lane of a group of four reads lane kLane of its group
+  return __builtin_amdgcn_mov_dpp(v, kLane * 0x55, 0xf, 0xf, false);
+}
+
+template <typename T>
+__device__ __forceinline__ void fetch_batch(const BatchInfo& bi, const PackedNode<T>* __restrict__ nodes,
+                                            const PackedTree* __restrict__ desc, int q, uint4 (&words)[kCopyWords],
+                                            int (&base)[kLaneTrees])
+{
+  constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
+  // the packed array is 16-byte aligned and batches start on 16-byte boundaries (see predict_tiled)
+  const uint4* src = reinterpret_cast<const uint4*>(nodes + bi.node_off);
+  const int n16    = (bi.total + kNodesPerWord - 1) / kNodesPerWord;
+#pragma unroll
+  for (int c = 0; c < kCopyWords; c++) {
+    const int i = threadIdx.x + c * kTileThreads;
+    words[c]    = src[i < n16 ? i : 0];
+  }
+#pragma unroll
+  for (int j = 0; j < kLaneTrees; j++) {
+    const int jj = q + kRowLanes * j;
+    base[j]      = desc[bi.first + (jj < bi.count ? jj : 0)].rel_off;  // lanes without a tree walk tree 0 again
+  }
+}
+
+template <typename T, bool kSingle>
+__global__ void __launch_bounds__(kTileThreads)
+  predict_tile_kernel(const T* __restrict__ X, int64_t n_rows, int F, int pitch, int n_batches,
+                      const BatchInfo* __restrict__ batches, const PackedTree* __restrict__ desc,
+                      const PackedNode<T>* __restrict__ nodes, int K, double* __restrict__ out)
+{
+  extern __shared__ unsigned char smem_raw[];
+  T* s_x = reinterpret_cast<T*>(smem_raw);
+  const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
+  PackedNode<T>* s_nodes = reinterpret_cast<PackedNode<T>*>(smem_raw + x_bytes);
+  uint4* s_words         = reinterpret_cast<uint4*>(smem_raw + x_bytes);
+  constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
+
+  const int64_t row0  = blockIdx.x * static_cast<int64_t>(kTileRows);
+  const int rows_here = static_cast<int>(min<int64_t>(kTileRows, n_rows - row0));
+  {
+    const T* src    = X + row0 * F;
+    const int total = rows_here * F;
+    if (sizeof(T) == 4 && (F & 3) == 0 && (reinterpret_cast<uintptr_t>(X) & 15) == 0) {
+      const float4* src4 = reinterpret_cast<const float4*>(src);
+      float* sx          = reinterpret_cast<float*>(s_x);
+      for (int i = threadIdx.x; i < total / 4; i += kTileThreads) {
+        const float4 v = src4[i];
+        const int e = i * 4, r = e / F, f = e - r * F;
+        float* d = sx + r * pitch + f;
+        d[0] = v.x;
+        d[1] = v.y;
+        d[2] = v.z;
+        d[3] = v.w;
+      }
+    } else {
+      for (int i = threadIdx.x; i < total; i += kTileThreads) {
+        const int r = i / F, f = i - r * F;
+        s_x[r * pitch + f] = src[i];
+      }
+    }
+  }
+  const int r      = threadIdx.x >> 2;
+  const int q      = threadIdx.x & 3;
+  const bool valid = r < rows_here;
+  const T* my_x    = s_x + (valid ? r : 0) * pitch;
+  constexpr int kAcc = kSingle ? 1 : kTileMaxK;
+  double acc[kAcc];
+#pragma unroll
+  for (int k = 0; k < kAcc; k++) acc[k] = 0.0;
+
+  // fetched one batch ahead: the batch descriptor, the nodes (as 16-byte words) and where this
+  // lane's trees start inside the batch
+  BatchInfo info_n = batches[0];
+  uint4 words_n[kCopyWords];
+  int base_n[kLaneTrees];
+  fetch_batch<T>(info_n, nodes, desc, q, words_n, base_n);
+  constexpr int kVal = kSingle ? kBatchTrees : 1;
+  double val[kVal];  // leaf values of the previous batch (single output)
+  int cnt_prev = 0;
+#pragma unroll
+  for (int jj = 0; jj < kVal; jj++) val[jj] = 0.0;
+
+  for (int b = 0; b < n_batches; b++) {
+    const BatchInfo info = info_n;
+    __syncthreads();  // the previous batch is no longer read; on the first pass: X tile complete
+    {
+      const int n16 = (info.total + kNodesPerWord - 1) / kNodesPerWord;
+#pragma unroll
+      for (int c = 0; c < kCopyWords; c++) {
+        const int i = threadIdx.x + c * kTileThreads;
+        if (i < n16) s_words[i] = words_n[c];
+      }
+    }
+    int base[kLaneTrees], pos[kLaneTrees];
+#pragma unroll
+    for (int j = 0; j < kLaneTrees; j++) {
+      base[j] = base_n[j];
+      pos[j]  = 0;
+    }
+    __syncthreads();
+    if (b + 1 < n_batches) {
+      info_n = batches[b + 1];
+      fetch_batch<T>(info_n, nodes, desc, q, words_n, base_n);
+    }
+    for (int s = 0; s < info.steps; s++) {
+#pragma unroll
+      for (int j = 0; j < kLaneTrees; j++) {
+        const PackedNode<T> nd = s_nodes[base[j] + pos[j]];
+        if constexpr (sizeof(T) == 4) {
+          const float xv = my_x[nd.feat_right & 0xffffu];
+          pos[j]         = static_cast<int>(nd.feat_right >> 16) - (xv <= nd.thr ? 1 : 0);
+        } else {
+          const double xv = my_x[nd.feat];
+          pos[j]          = nd.right - (xv <= nd.thr ? 1 : 0);
+        }
+      }
+    }
+    if constexpr (kSingle) {
+      // leaf values of the previous batch arrived while this one was walked: add them in tree order
+#pragma unroll
+      for (int jj = 0; jj < kBatchTrees; jj++)
+        if (jj < cnt_prev) acc[0] += val[jj];
+#pragma unroll
+      for (int jj = 0; jj < kBatchTrees; jj++) {
+        int p = 0;
+        if ((jj & 3) == 0) p = quad_broadcast<0>(pos[jj >> 2]);
+        if ((jj & 3) == 1) p = quad_broadcast<1>(pos[jj >> 2]);
+        if ((jj & 3) == 2) p = quad_broadcast<2>(pos[jj >> 2]);
+        if ((jj & 3) == 3) p = quad_broadcast<3>(pos[jj >> 2]);
+        val[jj] = jj < info.count ? desc[info.first + jj].leaf[p] : 0.0;
+      }
+      cnt_prev = info.count;
+    } else {
+#pragma unroll
+      for (int jj = 0; jj < kBatchTrees; jj++) {
+        int p = 0;
+        if ((jj & 3) == 0) p = quad_broadcast<0>(pos[jj >> 2]);
+        if ((jj & 3) == 1) p = quad_broadcast<1>(pos[jj >> 2]);
+        if ((jj & 3) == 2) p = quad_broadcast<2>(pos[jj >> 2]);
+        if ((jj & 3) == 3) p = quad_broadcast<3>(pos[jj >> 2]);
+        if (jj < info.count) {
+          const double* lf = desc[info.first + jj].leaf + static_cast<int64_t>(p) * K;
+#pragma unroll
+          for (int k = 0; k < kAcc; k++)
+            if (k < K) acc[k] += lf[k];
+        }
+      }
+    }
+  }
+  if constexpr (kSingle) {
+#pragma unroll
+    for (int jj = 0; jj < kBatchTrees; jj++)
+      if (jj < cnt_prev) acc[0] += val[jj];
+  }
+  if (valid && q == 0) {
+    double* o = out + (row0 + r) * K;
+#pragma unroll
+    for (int k = 0; k < kAcc; k++)
+      if (k < K) o[k] = acc[k];
+  }
+}
+
+size_t packed_bytes(int n_trees, int64_t total_nodes, size_t node_size)
+{
+  // tree descriptors, batch descriptors (at most one per tree), nodes (batches start on 16 bytes)
+  return ((static_cast<size_t>(n_trees) * sizeof(PackedTree) + 255) & ~size_t(255)) +
+         ((static_cast<size_t>(n_trees) * sizeof(BatchInfo) + 255) & ~size_t(255)) +
+         (static_cast<size_t>(total_nodes) + 2 * static_cast<size_t>(n_trees)) * node_size + 512;
+}
+
+// Returns LBT_OK and sets *done when the tiled path ran; leaves *done false when the shapes
+// do not fit it (then the caller takes the per-node path).
+template <typename T>
+int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees, const double* const* leaf,
+                  const int32_t* const* feature, const double* const* split, const int32_t* tree_nodes, int K,
+                  double* out, void* workspace, size_t workspace_bytes, bool* done)
+{
+  *done = false;
+  if (workspace == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
+  const int pitch      = F | 1;  // odd pitch: the rows of a wave start in different LDS banks
+  const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
+  if (x_bytes + 4096 > kTileLds) return LBT_OK;
+  constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
+  const int64_t node_cap = std::min<int64_t>(static_cast<int64_t>((kTileLds - x_bytes) / sizeof(PackedNode<T>)),
+                                             static_cast<int64_t>(kCopyWords) * kTileThreads * kNodesPerWord);
+  int64_t total_nodes = 0;
+  int max_nodes       = 0;
+  for (int i = 0; i < n_trees; i++) {
+    total_nodes += tree_nodes[i];
+    max_nodes = std::max(max_nodes, tree_nodes[i]);
+  }
+  if (max_nodes > node_cap || max_nodes > kMaxPackedNodes) return LBT_OK;
+  const size_t need = packed_bytes(n_trees, total_nodes, sizeof(PackedNode<T>));
+  if (workspace_bytes < need) {
+    set_error("predict workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
+    return LBT_ERR_WORKSPACE;
+  }
+  const size_t desc_bytes  = (static_cast<size_t>(n_trees) * sizeof(PackedTree) + 255) & ~size_t(255);
+  const size_t batch_bytes = (static_cast<size_t>(n_trees) * sizeof(BatchInfo) + 255) & ~size_t(255);
+  uintptr_t raw            = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255);
+  PackedTree* desc         = reinterpret_cast<PackedTree*>(raw);
+  BatchInfo* batches       = reinterpret_cast<BatchInfo*>(raw + desc_bytes);
+  PackedNode<T>* nodes     = reinterpret_cast<PackedNode<T>*>(raw + desc_bytes + batch_bytes);
+
+  // batches: consecutive trees, at most kBatchTrees, whose nodes fit the LDS share together
+  std::vector<BatchInfo> binfo;
+  std::vector<int64_t> node_off(n_trees);
+  std::vector<int32_t> rel_off(n_trees);
+  int64_t off = 0;
+  for (int t = 0; t < n_trees;) {
+    off = (off + kNodesPerWord - 1) / kNodesPerWord * kNodesPerWord;  // 16-byte aligned start
+    BatchInfo bi{};
+    bi.node_off = off;
+    bi.first    = t;
+    int64_t in_batch = 0;
+    while (t < n_trees && bi.count < kBatchTrees && in_batch + tree_nodes[t] <= node_cap) {
+      node_off[t] = off + in_batch;
+      rel_off[t]  = static_cast<int32_t>(in_batch);
+      int steps   = 0;
+      while (((int64_t(1) << (steps + 1)) - 1) < tree_nodes[t]) steps++;
+      bi.steps = std::max(bi.steps, steps);
+      in_batch += tree_nodes[t];
+      bi.count++;
+      t++;
+    }
+    bi.total = static_cast<int32_t>(in_batch);
+    off += in_batch;
+    binfo.push_back(bi);
+  }
+  ProfScope ps(LBT_PROF_PREDICT, stream, static_cast<double>(N) * (static_cast<double>(F) * sizeof(T) + K * 8.0));
+  for (int first = 0; first < n_trees; first += kPackTrees) {
+    PackBatch b{};
+    const int n = std::min(kPackTrees, n_trees - first);
+    int widest  = 1;
+    for (int i = 0; i < n; i++) {
+      b.t[i].leaf    = leaf[first + i];
+      b.t[i].feature = feature[first + i];
+      b.t[i].split   = split[first + i];
+      b.t[i].n_nodes = tree_nodes[first + i];
+      b.node_off[i]  = node_off[first + i];
+      b.rel_off[i]   = rel_off[first + i];
+      widest         = std::max(widest, tree_nodes[first + i]);
+    }
+    dim3 grid(static_cast<unsigned>((widest + 255) / 256), n);
+    pack_trees_kernel<T><<<grid, 256, 0, stream>>>(b, first, F, desc, nodes);
+  }
+  const int n_batches = static_cast<int>(binfo.size());
+  for (int first = 0; first < n_batches; first += kPackBatches) {
+    BatchTable tb{};
+    const int n = std::min(kPackBatches, n_batches - first);
+    for (int i = 0; i < n; i++) tb.b[i] = binfo[first + i];
+    write_batches_kernel<<<1, kPackBatches, 0, stream>>>(tb, first, n, batches);
+  }
+  static bool attr_set = false;
+  if (!attr_set) {
+    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(predict_tile_kernel<T, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kTileLds)));
+    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(predict_tile_kernel<T, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kTileLds)));
+    attr_set = true;
+  }
+  const unsigned tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
+  if (K == 1)
+    predict_tile_kernel<T, true><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
+                                                                            nodes, K, out);
+  else
+    predict_tile_kernel<T, false><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
+                                                                             nodes, K, out);
+  LBT_HIP(hipGetLastError());
+  *done = true;
+  return LBT_OK;
+}
+
 // ---- update
 
 __global__ void zero_doubles_kernel(double* a, int64_t n)
@@ -144,7 +539,7 @@ extern "C" {
 int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
                 int32_t n_trees, const double* const* leaf, const int32_t* const* feature,
                 const double* const* split, const int32_t* tree_nodes, int32_t n_outputs,
-                double* out)
+                double* out, void* workspace, size_t workspace_bytes)
 {
   LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
   LBT_REQUIRE(n_features >= 1 && n_outputs >= 1 && n_trees >= 0, "bad shape");
@@ -160,11 +555,26 @@ int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, in
       out, n_rows * n_outputs);
     return LBT_OK;
   }
-  if (x_dtype == LBT_F32)
+  bool done = false;
+  if (x_dtype == LBT_F32) {
+    LBT_TRY(lbt::predict_tiled<float>(s, static_cast<const float*>(X), n_rows, n_features, n_trees, leaf, feature,
+                                      split, tree_nodes, n_outputs, out, workspace, workspace_bytes, &done));
+    if (done) return LBT_OK;
     return lbt::predict_impl<float>(s, static_cast<const float*>(X), n_rows, n_features, n_trees, leaf,
                                     feature, split, tree_nodes, n_outputs, out);
+  }
+  LBT_TRY(lbt::predict_tiled<double>(s, static_cast<const double*>(X), n_rows, n_features, n_trees, leaf, feature,
+                                     split, tree_nodes, n_outputs, out, workspace, workspace_bytes, &done));
+  if (done) return LBT_OK;
   return lbt::predict_impl<double>(s, static_cast<const double*>(X), n_rows, n_features, n_trees, leaf,
                                    feature, split, tree_nodes, n_outputs, out);
+}
+
+size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t x_dtype)
+{
+  if (n_trees < 0 || total_nodes < 0 || (x_dtype != LBT_F32 && x_dtype != LBT_F64)) return 0;
+  return lbt::packed_bytes(n_trees, total_nodes,
+                           x_dtype == LBT_F32 ? sizeof(lbt::PackedNode<float>) : sizeof(lbt::PackedNode<double>));
 }
 
 size_t lbt_update_tree_workspace_bytes(int64_t n_rows, int32_t n_outputs, int32_t n_nodes)

@@ -88,7 +88,9 @@ def _load():
                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(BuildTaps)]
     lib.lbt_predict.restype = C.c_int
     lib.lbt_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_void_p,
-                                C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]
+                                C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_predict_workspace_bytes.restype = C.c_size_t
+    lib.lbt_predict_workspace_bytes.argtypes = [C.c_int32, C.c_int64, C.c_int32]
     lib.lbt_update_tree_workspace_bytes.restype = C.c_size_t
     lib.lbt_update_tree_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     lib.lbt_update_tree.restype = C.c_int
@@ -107,6 +109,7 @@ lib = _load()
 
 EXPORTS = [
     "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_predict",
+    "lbt_predict_workspace_bytes",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",
 ]

@@ -144,7 +144,7 @@ def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0
     return r
 
 
-def predict(X, trees, n_outputs):
+def predict(X, trees, n_outputs, tiled=True):
     """PREDICT (legateboost/models/tree.py:245-280). trees: sequence of
     (leaf_value [nodes,K] f64, feature [nodes] i32, split_value [nodes] f64) CUDA tensors."""
     X = _check_x(X)
@@ -164,8 +164,14 @@ def predict(X, trees, n_outputs):
             raise _lib.LbtError("tree %d has inconsistent shapes" % i)
         keep.append((lv, ft, sp))
         leaf_p[i], feat_p[i], split_p[i], nodes[i] = lv.data_ptr(), ft.data_ptr(), sp.data_ptr(), ft.shape[0]
+    total_nodes = sum(int(nodes[i]) for i in range(nt))
+    ws = None
+    if tiled:
+        ws = torch.empty(int(_lib.lib.lbt_predict_workspace_bytes(nt, total_nodes, _DT[X.dtype])), dtype=torch.uint8,
+                         device=X.device)
     rc = _lib.lib.lbt_predict(_stream(), X.data_ptr(), _DT[X.dtype], n, f, nt, leaf_p, feat_p, split_p, nodes,
-                              n_outputs, out.data_ptr())
+                              n_outputs, out.data_ptr(), ws.data_ptr() if ws is not None else None,
+                              ws.numel() if ws is not None else 0)
     _lib.check(rc)
     return out
 
