@@ -108,9 +108,9 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
                    double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
                    void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
 
-/* Device scratch for lbt_predict: room for the ensemble packed into one node array
- * (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
-size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t x_dtype);
+/* Device scratch for lbt_predict: room for the ensemble packed into one node array and one
+ * leaf array (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
+size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype);
 
 /*
  * PredictTask::gpu_variant (src/models/tree/predict.cu:26-91).

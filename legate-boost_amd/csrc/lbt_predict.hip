@@ -104,7 +104,7 @@ int predict_impl(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
 // step costs two LDS reads and no trip to the L2. Four lanes share a row and take every fourth
 // tree of the batch, five trees each, interleaved for latency. The nodes of the next batch are
 // fetched into registers while the current one is walked, and the leaf values of a batch are
-// fetched while the next one is walked. They are added in tree order, so a row's sum is formed
+// fetched (from a packed copy) while the next one is walked. They are added in tree order, so a row's sum is formed
 // exactly as the per-tree launches of the reference form it.
 
 template <typename T>
@@ -175,7 +175,8 @@ __device__ inline float round_down_to_float(double d)
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-  pack_trees_kernel(PackBatch b, int first_tree, int F, PackedTree* desc, PackedNode<T>* nodes)
+  pack_trees_kernel(PackBatch b, int first_tree, int F, int K, PackedTree* desc, PackedNode<T>* nodes,
+                    double* leaves)
 {
   const TreeRef tr = b.t[blockIdx.y];
   const int i      = blockIdx.x * 256 + threadIdx.x;
@@ -187,6 +188,9 @@ __global__ void __launch_bounds__(256)
     desc[first_tree + blockIdx.y] = d;
   }
   if (i >= tr.n_nodes) return;
+  // leaf values move along, indexed like the nodes
+  for (int k = 0; k < K; k++)
+    leaves[(b.node_off[blockIdx.y] + i) * K + k] = tr.leaf[static_cast<int64_t>(i) * K + k];
   int ft = tr.feature[i];
   // a node whose children would lie past the arrays, or whose feature does not exist, ends the walk
   const bool is_leaf = ft < 0 || ft >= F || 2 * static_cast<int64_t>(i) + 2 >= tr.n_nodes;
@@ -216,39 +220,98 @@ __device__ inline int quad_broadcast(int v)
   // every lane of a group of four reads lane kLane of its group
   return __builtin_amdgcn_mov_dpp(v, kLane * 0x55, 0xf, 0xf, false);
 }
+template <int kLane>
+__device__ inline double quad_broadcast(double v)
+{
+  const long long bits = __double_as_longlong(v);
+  const int lo = quad_broadcast<kLane>(static_cast<int>(bits));
+  const int hi = quad_broadcast<kLane>(static_cast<int>(bits >> 32));
+  return __longlong_as_double((static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
+}
+// value of tree jj of a batch, held by lane jj % 4 of the row's four lanes in slot jj / 4
+template <int jj, typename V>
+__device__ inline V from_owner(const V (&slots)[5])
+{
+  return quad_broadcast<jj & 3>(slots[jj >> 2]);
+}
+
+// What is fetched one batch ahead: the nodes as 16-byte words and where this lane's trees start
+// inside the batch.
+typedef unsigned int Word16 __attribute__((ext_vector_type(4)));  // plain vector: stays in registers
+struct Prefetched {
+  Word16 words[kCopyWords];
+  int base[kLaneTrees];
+};
 
 template <typename T>
-__device__ __forceinline__ void fetch_batch(const BatchInfo& bi, const PackedNode<T>* __restrict__ nodes,
-                                            const PackedTree* __restrict__ desc, int q, uint4 (&words)[kCopyWords],
-                                            int (&base)[kLaneTrees])
+__device__ __forceinline__ Prefetched fetch_batch(const BatchInfo& bi, const PackedNode<T>* __restrict__ nodes,
+                                                  const PackedTree* __restrict__ desc, int q)
 {
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
+  Prefetched pf;
   // the packed array is 16-byte aligned and batches start on 16-byte boundaries (see predict_tiled)
-  const uint4* src = reinterpret_cast<const uint4*>(nodes + bi.node_off);
-  const int n16    = (bi.total + kNodesPerWord - 1) / kNodesPerWord;
+  const Word16* src = reinterpret_cast<const Word16*>(nodes + bi.node_off);
+  const int n16     = (bi.total + kNodesPerWord - 1) / kNodesPerWord;
 #pragma unroll
   for (int c = 0; c < kCopyWords; c++) {
     const int i = threadIdx.x + c * kTileThreads;
-    words[c]    = src[i < n16 ? i : 0];
+    pf.words[c] = src[i < n16 ? i : 0];
   }
 #pragma unroll
   for (int j = 0; j < kLaneTrees; j++) {
     const int jj = q + kRowLanes * j;
-    base[j]      = desc[bi.first + (jj < bi.count ? jj : 0)].rel_off;  // lanes without a tree walk tree 0 again
+    pf.base[j]   = desc[bi.first + (jj < bi.count ? jj : 0)].rel_off;  // lanes without a tree walk tree 0 again
   }
+  return pf;
+}
+
+template <int jj>
+__device__ __forceinline__ void add_in_order_from(double& acc, const double (&val)[kLaneTrees], int cnt)
+{
+  if constexpr (jj < kBatchTrees) {
+    const double v = from_owner<jj>(val);
+    if (jj < cnt) acc += v;
+    add_in_order_from<jj + 1>(acc, val, cnt);
+  }
+}
+__device__ __forceinline__ void add_in_order(double& acc, const double (&val)[kLaneTrees], int cnt)
+{
+  add_in_order_from<0>(acc, val, cnt);
+}
+template <int kAcc, int jj>
+__device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[kLaneTrees], int cnt,
+                                                const double* __restrict__ batch_leaves, int K)
+{
+  if constexpr (jj < kBatchTrees) {
+    const int p = from_owner<jj>(at);
+    if (jj < cnt) {
+      const double* lf = batch_leaves + static_cast<int64_t>(p) * K;
+#pragma unroll
+      for (int k = 0; k < kAcc; k++)
+        if (k < K) acc[k] += lf[k];
+    }
+    add_leaves_from<kAcc, jj + 1>(acc, at, cnt, batch_leaves, K);
+  }
+}
+template <int kAcc>
+__device__ __forceinline__ void add_leaves_in_order(double (&acc)[kAcc], const int (&at)[kLaneTrees], int cnt,
+                                                    const double* __restrict__ batch_leaves, int K)
+{
+  add_leaves_from<kAcc, 0>(acc, at, cnt, batch_leaves, K);
 }
 
 template <typename T, bool kSingle>
 __global__ void __launch_bounds__(kTileThreads)
   predict_tile_kernel(const T* __restrict__ X, int64_t n_rows, int F, int pitch, int n_batches,
                       const BatchInfo* __restrict__ batches, const PackedTree* __restrict__ desc,
-                      const PackedNode<T>* __restrict__ nodes, int K, double* __restrict__ out)
+                      const PackedNode<T>* __restrict__ nodes, const double* __restrict__ leaves, int K,
+                      double* __restrict__ out)
 {
   extern __shared__ unsigned char smem_raw[];
   T* s_x = reinterpret_cast<T*>(smem_raw);
   const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
   PackedNode<T>* s_nodes = reinterpret_cast<PackedNode<T>*>(smem_raw + x_bytes);
-  uint4* s_words         = reinterpret_cast<uint4*>(smem_raw + x_bytes);
+  Word16* s_words        = reinterpret_cast<Word16*>(smem_raw + x_bytes);
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
 
   const int64_t row0  = blockIdx.x * static_cast<int64_t>(kTileRows);
@@ -287,14 +350,11 @@ __global__ void __launch_bounds__(kTileThreads)
   // fetched one batch ahead: the batch descriptor, the nodes (as 16-byte words) and where this
   // lane's trees start inside the batch
   BatchInfo info_n = batches[0];
-  uint4 words_n[kCopyWords];
-  int base_n[kLaneTrees];
-  fetch_batch<T>(info_n, nodes, desc, q, words_n, base_n);
-  constexpr int kVal = kSingle ? kBatchTrees : 1;
-  double val[kVal];  // leaf values of the previous batch (single output)
+  Prefetched pf = fetch_batch<T>(info_n, nodes, desc, q);
+  double val[kLaneTrees];  // single output: leaf values of this lane's trees of the previous batch
   int cnt_prev = 0;
 #pragma unroll
-  for (int jj = 0; jj < kVal; jj++) val[jj] = 0.0;
+  for (int j = 0; j < kLaneTrees; j++) val[j] = 0.0;
 
   for (int b = 0; b < n_batches; b++) {
     const BatchInfo info = info_n;
@@ -304,19 +364,19 @@ __global__ void __launch_bounds__(kTileThreads)
 #pragma unroll
       for (int c = 0; c < kCopyWords; c++) {
         const int i = threadIdx.x + c * kTileThreads;
-        if (i < n16) s_words[i] = words_n[c];
+        if (i < n16) s_words[i] = pf.words[c];
       }
     }
     int base[kLaneTrees], pos[kLaneTrees];
 #pragma unroll
     for (int j = 0; j < kLaneTrees; j++) {
-      base[j] = base_n[j];
+      base[j] = pf.base[j];
       pos[j]  = 0;
     }
     __syncthreads();
     if (b + 1 < n_batches) {
       info_n = batches[b + 1];
-      fetch_batch<T>(info_n, nodes, desc, q, words_n, base_n);
+      pf = fetch_batch<T>(info_n, nodes, desc, q);
     }
     for (int s = 0; s < info.steps; s++) {
 #pragma unroll
@@ -332,42 +392,20 @@ __global__ void __launch_bounds__(kTileThreads)
       }
     }
     if constexpr (kSingle) {
-      // leaf values of the previous batch arrived while this one was walked: add them in tree order
+      // leaf values of the previous batch arrived while this one was walked: every lane of the
+      // four forms the same sum, in tree order
+      add_in_order(acc[0], val, cnt_prev);
 #pragma unroll
-      for (int jj = 0; jj < kBatchTrees; jj++)
-        if (jj < cnt_prev) acc[0] += val[jj];
-#pragma unroll
-      for (int jj = 0; jj < kBatchTrees; jj++) {
-        int p = 0;
-        if ((jj & 3) == 0) p = quad_broadcast<0>(pos[jj >> 2]);
-        if ((jj & 3) == 1) p = quad_broadcast<1>(pos[jj >> 2]);
-        if ((jj & 3) == 2) p = quad_broadcast<2>(pos[jj >> 2]);
-        if ((jj & 3) == 3) p = quad_broadcast<3>(pos[jj >> 2]);
-        val[jj] = jj < info.count ? desc[info.first + jj].leaf[p] : 0.0;
-      }
+      for (int j = 0; j < kLaneTrees; j++) val[j] = leaves[info.node_off + base[j] + pos[j]];
       cnt_prev = info.count;
     } else {
+      int at[kLaneTrees];
 #pragma unroll
-      for (int jj = 0; jj < kBatchTrees; jj++) {
-        int p = 0;
-        if ((jj & 3) == 0) p = quad_broadcast<0>(pos[jj >> 2]);
-        if ((jj & 3) == 1) p = quad_broadcast<1>(pos[jj >> 2]);
-        if ((jj & 3) == 2) p = quad_broadcast<2>(pos[jj >> 2]);
-        if ((jj & 3) == 3) p = quad_broadcast<3>(pos[jj >> 2]);
-        if (jj < info.count) {
-          const double* lf = desc[info.first + jj].leaf + static_cast<int64_t>(p) * K;
-#pragma unroll
-          for (int k = 0; k < kAcc; k++)
-            if (k < K) acc[k] += lf[k];
-        }
-      }
+      for (int j = 0; j < kLaneTrees; j++) at[j] = base[j] + pos[j];
+      add_leaves_in_order<kAcc>(acc, at, info.count, leaves + info.node_off * K, K);
     }
   }
-  if constexpr (kSingle) {
-#pragma unroll
-    for (int jj = 0; jj < kBatchTrees; jj++)
-      if (jj < cnt_prev) acc[0] += val[jj];
-  }
+  if constexpr (kSingle) add_in_order(acc[0], val, cnt_prev);
   if (valid && q == 0) {
     double* o = out + (row0 + r) * K;
 #pragma unroll
@@ -376,12 +414,17 @@ __global__ void __launch_bounds__(kTileThreads)
   }
 }
 
-size_t packed_bytes(int n_trees, int64_t total_nodes, size_t node_size)
+size_t padded_nodes(int n_trees, int64_t total_nodes)
 {
-  // tree descriptors, batch descriptors (at most one per tree), nodes (batches start on 16 bytes)
+  return static_cast<size_t>(total_nodes) + 2 * static_cast<size_t>(n_trees);  // batches start on 16 bytes
+}
+size_t packed_bytes(int n_trees, int64_t total_nodes, int K, size_t node_size)
+{
+  // tree descriptors, batch descriptors (at most one per tree), nodes, leaf values
   return ((static_cast<size_t>(n_trees) * sizeof(PackedTree) + 255) & ~size_t(255)) +
          ((static_cast<size_t>(n_trees) * sizeof(BatchInfo) + 255) & ~size_t(255)) +
-         (static_cast<size_t>(total_nodes) + 2 * static_cast<size_t>(n_trees)) * node_size + 512;
+         ((padded_nodes(n_trees, total_nodes) * node_size + 255) & ~size_t(255)) +
+         padded_nodes(n_trees, total_nodes) * static_cast<size_t>(K) * sizeof(double) + 512;
 }
 
 // Returns LBT_OK and sets *done when the tiled path ran; leaves *done false when the shapes
@@ -406,7 +449,7 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
     max_nodes = std::max(max_nodes, tree_nodes[i]);
   }
   if (max_nodes > node_cap || max_nodes > kMaxPackedNodes) return LBT_OK;
-  const size_t need = packed_bytes(n_trees, total_nodes, sizeof(PackedNode<T>));
+  const size_t need = packed_bytes(n_trees, total_nodes, K, sizeof(PackedNode<T>));
   if (workspace_bytes < need) {
     set_error("predict workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
     return LBT_ERR_WORKSPACE;
@@ -417,6 +460,8 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   PackedTree* desc         = reinterpret_cast<PackedTree*>(raw);
   BatchInfo* batches       = reinterpret_cast<BatchInfo*>(raw + desc_bytes);
   PackedNode<T>* nodes     = reinterpret_cast<PackedNode<T>*>(raw + desc_bytes + batch_bytes);
+  const size_t node_bytes  = (padded_nodes(n_trees, total_nodes) * sizeof(PackedNode<T>) + 255) & ~size_t(255);
+  double* leaves           = reinterpret_cast<double*>(raw + desc_bytes + batch_bytes + node_bytes);
 
   // batches: consecutive trees, at most kBatchTrees, whose nodes fit the LDS share together
   std::vector<BatchInfo> binfo;
@@ -458,7 +503,7 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
       widest         = std::max(widest, tree_nodes[first + i]);
     }
     dim3 grid(static_cast<unsigned>((widest + 255) / 256), n);
-    pack_trees_kernel<T><<<grid, 256, 0, stream>>>(b, first, F, desc, nodes);
+    pack_trees_kernel<T><<<grid, 256, 0, stream>>>(b, first, F, K, desc, nodes, leaves);
   }
   const int n_batches = static_cast<int>(binfo.size());
   for (int first = 0; first < n_batches; first += kPackBatches) {
@@ -478,10 +523,10 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   const unsigned tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
   if (K == 1)
     predict_tile_kernel<T, true><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
-                                                                            nodes, K, out);
+                                                                            nodes, leaves, K, out);
   else
     predict_tile_kernel<T, false><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
-                                                                             nodes, K, out);
+                                                                             nodes, leaves, K, out);
   LBT_HIP(hipGetLastError());
   *done = true;
   return LBT_OK;
@@ -570,10 +615,10 @@ int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, in
                                    feature, split, tree_nodes, n_outputs, out);
 }
 
-size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t x_dtype)
+size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype)
 {
-  if (n_trees < 0 || total_nodes < 0 || (x_dtype != LBT_F32 && x_dtype != LBT_F64)) return 0;
-  return lbt::packed_bytes(n_trees, total_nodes,
+  if (n_trees < 0 || total_nodes < 0 || n_outputs < 1 || (x_dtype != LBT_F32 && x_dtype != LBT_F64)) return 0;
+  return lbt::packed_bytes(n_trees, total_nodes, n_outputs,
                            x_dtype == LBT_F32 ? sizeof(lbt::PackedNode<float>) : sizeof(lbt::PackedNode<double>));
 }
 

@@ -138,9 +138,16 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
     split.push_back(dense_in<double, 1>(context.input(i + 2).data(), &ss));
     nodes.push_back(static_cast<int32_t>(fs.hi[0] - fs.lo[0] + 1));
   }
+  // scratch for the packed ensemble (the task class gains with_has_allocations(true))
+  int64_t total_nodes = 0;
+  for (int32_t n : nodes) total_nodes += n;
+  const size_t ws_bytes =
+    lbt_predict_workspace_bytes(static_cast<int>(leaf.size()), total_nodes, outputs, dtype);
+  auto workspace = legate::create_buffer<int8_t>(ws_bytes, legate::Memory::GPU_FB_MEM, 256);
   check(lbt_predict(context.get_task_stream(), X, dtype, rows, static_cast<int>(xs.hi[1] - xs.lo[1] + 1),
                     static_cast<int>(leaf.size()), leaf.data(), feature.data(), split.data(), nodes.data(), outputs,
-                    out));
+                    out, workspace.ptr(0), ws_bytes));
+  // the buffer is task-scoped: Legate frees it once the work enqueued on the task stream is done
 }
 
 /*static*/ void UpdateTreeTask::gpu_variant(legate::TaskContext context)

@@ -90,7 +90,7 @@ def _load():
     lib.lbt_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.lbt_predict_workspace_bytes.restype = C.c_size_t
-    lib.lbt_predict_workspace_bytes.argtypes = [C.c_int32, C.c_int64, C.c_int32]
+    lib.lbt_predict_workspace_bytes.argtypes = [C.c_int32, C.c_int64, C.c_int32, C.c_int32]
     lib.lbt_update_tree_workspace_bytes.restype = C.c_size_t
     lib.lbt_update_tree_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32]
     lib.lbt_update_tree.restype = C.c_int

@@ -167,7 +167,7 @@ def predict(X, trees, n_outputs, tiled=True):
     total_nodes = sum(int(nodes[i]) for i in range(nt))
     ws = None
     if tiled:
-        ws = torch.empty(int(_lib.lib.lbt_predict_workspace_bytes(nt, total_nodes, _DT[X.dtype])), dtype=torch.uint8,
+        ws = torch.empty(int(_lib.lib.lbt_predict_workspace_bytes(nt, total_nodes, n_outputs, _DT[X.dtype])), dtype=torch.uint8,
                          device=X.device)
     rc = _lib.lib.lbt_predict(_stream(), X.data_ptr(), _DT[X.dtype], n, f, nt, leaf_p, feat_p, split_p, nodes,
                               n_outputs, out.data_ptr(), ws.data_ptr() if ws is not None else None,
