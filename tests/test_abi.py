@@ -44,6 +44,10 @@ def test_workspace_query():
     assert q(1000, 32, 1, 40, 256, _lib.LBT_F32, 0) == 0
     assert q(1000, 32, 1, 6, 256, 7, 0) == 0
     assert _lib.lib.lbt_update_tree_workspace_bytes(1000, 2, 127) >= 127 * 2 * 16
+    # packed ensemble: 8 bytes per node for float X plus the leaf values
+    pw = _lib.lib.lbt_predict_workspace_bytes(1000, 511000, 1, _lib.LBT_F32)
+    assert 511000 * 16 <= pw < 511000 * 16 + (1 << 20)
+    assert _lib.lib.lbt_predict_workspace_bytes(10, 100, 0, _lib.LBT_F32) == 0
 
 
 def test_bad_arguments_are_rejected_without_a_gpu():
@@ -66,7 +70,7 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     rc = _lib.lib.lbt_build_tree(None, one, 5, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one, one, one,
                                  one, 1 << 20, None)
     assert rc == -1
-    rc = _lib.lib.lbt_predict(None, one, 9, 10, 2, 0, None, None, None, None, 1, one)
+    rc = _lib.lib.lbt_predict(None, one, 9, 10, 2, 0, None, None, None, None, 1, one, None, 0)
     assert rc == -1
     with pytest.raises(_lib.LbtError):
         _lib.check(rc)
