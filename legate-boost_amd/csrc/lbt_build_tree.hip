@@ -1058,28 +1058,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       uniq, S, L.row_pointers, static_cast<T*>(L.proposals), L.bin_feature);
     LBT_HIP(hipMemcpyAsync(rp.data(), L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
   }
-  LBT_HIP(hipStreamSynchronize(stream));
-  const int B = rp[F];
-  proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
-    static_cast<const T*>(L.proposals), B, L.proposals_d);
-
-  HistSetup hs;
-  hs.groups     = L.groups;
-  hs.sgroups    = L.sgroups;
-  hs.tables     = L.tables;
-  hs.cell_lo    = L.cell_lo;
-  hs.cell_invw  = L.cell_invw;
-  hs.tile_start = L.tile_start;
-  hs.tiles      = L.tiles;
-  hs.binned     = L.binned;
-  hs.binned_capacity = L.binned_bytes;
-  hs.bin_base   = L.bin_base;
-  hs.bin_stride = L.bin_stride;
-  hs.bin_tail   = L.bin_tail;
-  hs.rec        = L.rec;
-  hs.meta       = L.meta;
-  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
-
   // ---- quantiser
   {
     ProfScope ps(LBT_PROF_QUANTISE, stream, static_cast<double>(N) * K * (16 + 16 + 8));
@@ -1107,6 +1085,38 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   // ---- positions and histogram cache (TreeBuilder ctor, build_tree.cu:997-1017)
   fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.pos[0], N);
   init_seg_kernel<<<1, 64, 0, stream>>>(L.seg[0], static_cast<int32_t>(N));
+  static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
+  if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
+
+  // the one host wait before the levels: the bin counts decide the feature groups, and a
+  // gradient that does not fit 32 bits ends the call. The quantiser above keeps the GPU busy
+  // while the host waits.
+  LBT_HIP(hipStreamSynchronize(stream));
+  if (h_qstats[1] != 0) {
+    set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
+    return LBT_ERR_UNSUPPORTED;
+  }
+  const int B = rp[F];
+  proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
+    static_cast<const T*>(L.proposals), B, L.proposals_d);
+
+  HistSetup hs;
+  hs.groups     = L.groups;
+  hs.sgroups    = L.sgroups;
+  hs.tables     = L.tables;
+  hs.cell_lo    = L.cell_lo;
+  hs.cell_invw  = L.cell_invw;
+  hs.tile_start = L.tile_start;
+  hs.tiles      = L.tiles;
+  hs.binned     = L.binned;
+  hs.binned_capacity = L.binned_bytes;
+  hs.bin_base   = L.bin_base;
+  hs.bin_stride = L.bin_stride;
+  hs.bin_tail   = L.bin_tail;
+  hs.rec        = L.rec;
+  hs.meta       = L.meta;
+  LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
+
   const uint64_t max_bytes = prm.hist_cache_bytes > 0 ? static_cast<uint64_t>(prm.hist_cache_bytes) : 1000000000ULL;
   const uint64_t bytes_per_node = static_cast<uint64_t>(K) * B * 16ULL;
   uint64_t max_histogram_nodes  = std::max<uint64_t>(1, max_bytes / bytes_per_node);
@@ -1133,15 +1143,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     return LBT_OK;
   };
   LBT_TRY(zero_hist(hv.node_begin, hv.node_end));
-  static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
-  if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
-
-  LBT_HIP(hipStreamSynchronize(stream));
-  if (h_qstats[1] != 0) {
-    set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
-    return LBT_ERR_UNSUPPORTED;
-  }
-
   int cur_pos = 0, cur_seg = 0;
   // the feature-major bins serve the position updates of levels 0 .. max_depth-2
   const bool use_bins_t = hs.binned != nullptr && L.bins_t != nullptr;

@@ -1214,7 +1214,11 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   auto hist_bytes = [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; };
 
   // search groups: as few as the LDS allows with the smallest table ...
-  std::vector<int32_t> sgroups;
+  // the host arrays below feed asynchronous copies: they persist until the thread's next call,
+  // which starts after this one has synchronised the stream
+  static thread_local std::vector<int32_t> sgroups, groups, stride, tail;
+  static thread_local std::vector<int64_t> base;
+  static thread_local std::vector<RecInfo> rec;
   const size_t search_budget = kLdsBudget - 64;  // room for the slack entries and alignment
   size_t budget              = search_budget;
   for (;;) {
@@ -1242,10 +1246,10 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   hs.rpp       = rows_per_pass(sgroups, vec);
   LBT_HIP(hipMemcpyAsync(hs.sgroups, sgroups.data(), sizeof(int32_t) * sgroups.size(), hipMemcpyHostToDevice, stream));
 
-  std::vector<int32_t> groups;
-  std::vector<int64_t> base(F);
-  std::vector<int32_t> stride(F), tail(F, 0);
-  std::vector<RecInfo> rec;
+  base.assign(F, 0);
+  stride.assign(F, 0);
+  tail.assign(F, 0);
+  rec.clear();
   if (!cached) {
     // one kernel searches and accumulates: the search groups are the histogram groups
     groups       = sgroups;
@@ -1300,8 +1304,6 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     LBT_HIP(hipMemcpyAsync(hs.bin_stride, stride.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
     LBT_HIP(hipMemcpyAsync(hs.bin_tail, tail.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
   }
-  // the host vectors must outlive the asynchronous copies
-  LBT_HIP(hipStreamSynchronize(stream));
   ProfScope ps(LBT_PROF_PROPOSALS, stream);
   if (is_f64)
     build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,
