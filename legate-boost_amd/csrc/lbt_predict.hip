@@ -540,27 +540,85 @@ __global__ void zero_doubles_kernel(double* a, int64_t n)
   if (i < n) a[i] = 0.0;
 }
 
-// every node on a row's path receives the row's (g,h) (update_tree.cc:76-90)
-template <typename T>
-__global__ void __launch_bounds__(kThreads)
-  update_accumulate_kernel(const T* X, int64_t n_rows, int F, const double* g, const double* h, int K,
-                           const int32_t* feature, const double* split, int n_nodes, double* G, double* H)
+// Every node on a row's path receives the row's (g, h) (update_tree.cc:76-90). The sums of an
+// inner node are the sums of its children, so a row adds to the node it stops in only and
+// propagate_sums_kernel fills in the rest. A workgroup collects its rows in an LDS copy of the
+// node sums (when that fits) and adds the copy to the global sums once.
+constexpr int kUpdateThreads = 256;
+constexpr int kUpdateLdsDoubles = 8192;  // 64 KB
+
+template <typename T, bool kUseLds>
+__global__ void __launch_bounds__(kUpdateThreads)
+  update_accumulate_kernel(const T* __restrict__ X, int64_t n_rows, int F, const double* __restrict__ g,
+                           const double* __restrict__ h, int K, const int32_t* __restrict__ feature,
+                           const double* __restrict__ split, int n_nodes, double* G, double* H)
 {
-  const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
-  if (row >= n_rows) return;
-  const T* xrow = X + row * F;
-  int pos       = 0;
-  for (int depth = 0; depth < 100; depth++) {
-    for (int k = 0; k < K; k++) {
-      atomicAdd(&G[static_cast<int64_t>(pos) * K + k], g[row * K + k]);
-      atomicAdd(&H[static_cast<int64_t>(pos) * K + k], h[row * K + k]);
+  __shared__ double s_sum[kUseLds ? kUpdateLdsDoubles : 1];
+  const int n_sums = n_nodes * K;
+  if constexpr (kUseLds) {
+    for (int i = threadIdx.x; i < 2 * n_sums; i += kUpdateThreads) s_sum[i] = 0.0;
+    __syncthreads();
+  }
+  for (int64_t row = blockIdx.x * static_cast<int64_t>(kUpdateThreads) + threadIdx.x; row < n_rows;
+       row += static_cast<int64_t>(gridDim.x) * kUpdateThreads) {
+    const T* xrow = X + row * F;
+    int pos       = 0;
+    for (int depth = 0; depth < 100; depth++) {
+      const int ft = feature[pos];
+      if (ft == -1) break;
+      const double xv = static_cast<double>(xrow[ft]);
+      const int next  = xv <= split[pos] ? 2 * pos + 1 : 2 * pos + 2;
+      if (next >= n_nodes) break;
+      pos = next;
     }
-    int ft = feature[pos];
-    if (ft == -1) break;
-    double xv = static_cast<double>(xrow[ft]);
-    int next  = xv <= split[pos] ? 2 * pos + 1 : 2 * pos + 2;
-    if (next >= n_nodes) break;
-    pos = next;
+    for (int k = 0; k < K; k++) {
+      const double gv = g[row * K + k], hv = h[row * K + k];
+      if constexpr (kUseLds) {
+        unsafeAtomicAdd(&s_sum[pos * K + k], gv);
+        unsafeAtomicAdd(&s_sum[n_sums + pos * K + k], hv);
+      } else {
+        unsafeAtomicAdd(&G[static_cast<int64_t>(pos) * K + k], gv);
+        unsafeAtomicAdd(&H[static_cast<int64_t>(pos) * K + k], hv);
+      }
+    }
+  }
+  if constexpr (kUseLds) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_sums; i += kUpdateThreads) {
+      const double gv = s_sum[i], hv = s_sum[n_sums + i];
+      if (gv != 0.0) unsafeAtomicAdd(&G[i], gv);
+      if (hv != 0.0) unsafeAtomicAdd(&H[i], hv);
+    }
+  }
+}
+
+// sums of inner nodes, deepest level first: a node that leads on (the walk above leaves it)
+// adds what its two children hold
+__global__ void __launch_bounds__(1024)
+  propagate_sums_kernel(const int32_t* __restrict__ feature, int n_nodes, int K, double* G, double* H)
+{
+  int depth = 0;
+  while (((int64_t(1) << (depth + 1)) - 1) < n_nodes) depth++;
+  for (int d = depth - 1; d >= 0; d--) {
+    const int64_t first = (int64_t(1) << d) - 1, count = int64_t(1) << d;
+    for (int64_t i = threadIdx.x; i < count * K; i += blockDim.x) {
+      const int64_t node = first + i / K;
+      const int k        = static_cast<int>(i % K);
+      if (node < n_nodes && feature[node] != -1) {
+        double gs = 0.0, hs = 0.0;
+        if (2 * node + 1 < n_nodes) {
+          gs += G[(2 * node + 1) * K + k];
+          hs += H[(2 * node + 1) * K + k];
+        }
+        if (2 * node + 2 < n_nodes) {
+          gs += G[(2 * node + 2) * K + k];
+          hs += H[(2 * node + 2) * K + k];
+        }
+        G[node * K + k] += gs;
+        H[node * K + k] += hs;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -651,13 +709,26 @@ int lbt_update_tree(void* stream, const void* X, int32_t x_dtype, int64_t n_rows
   lbt::ProfScope ps(LBT_PROF_OTHER, s);
   lbt::zero_doubles_kernel<<<static_cast<unsigned>((2 * n + 255) / 256), 256, 0, s>>>(G, 2 * n);
   if (n_rows > 0) {
-    const unsigned grid = static_cast<unsigned>((n_rows + 255) / 256);
-    if (x_dtype == LBT_F32)
-      lbt::update_accumulate_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(X), n_rows, n_features,
-                                                                g, h, n_outputs, feature, split, n_nodes, G, H);
-    else
-      lbt::update_accumulate_kernel<double><<<grid, 256, 0, s>>>(static_cast<const double*>(X), n_rows, n_features,
-                                                                 g, h, n_outputs, feature, split, n_nodes, G, H);
+    const unsigned grid = static_cast<unsigned>(std::min<int64_t>((n_rows + 255) / 256, 4096));
+    const bool lds      = 2 * n <= lbt::kUpdateLdsDoubles;
+    if (x_dtype == LBT_F32) {
+      const float* Xf = static_cast<const float*>(X);
+      if (lds)
+        lbt::update_accumulate_kernel<float, true><<<grid, 256, 0, s>>>(Xf, n_rows, n_features, g, h, n_outputs,
+                                                                        feature, split, n_nodes, G, H);
+      else
+        lbt::update_accumulate_kernel<float, false><<<grid, 256, 0, s>>>(Xf, n_rows, n_features, g, h, n_outputs,
+                                                                         feature, split, n_nodes, G, H);
+    } else {
+      const double* Xd = static_cast<const double*>(X);
+      if (lds)
+        lbt::update_accumulate_kernel<double, true><<<grid, 256, 0, s>>>(Xd, n_rows, n_features, g, h, n_outputs,
+                                                                         feature, split, n_nodes, G, H);
+      else
+        lbt::update_accumulate_kernel<double, false><<<grid, 256, 0, s>>>(Xd, n_rows, n_features, g, h, n_outputs,
+                                                                          feature, split, n_nodes, G, H);
+    }
+    lbt::propagate_sums_kernel<<<1, 1024, 0, s>>>(feature, n_nodes, n_outputs, G, H);
   }
   lbt::update_leaves_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, s>>>(
     G, H, n, l1_regularization, l2_regularization, leaf_out, hessian_out);
