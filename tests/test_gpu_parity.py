@@ -29,6 +29,9 @@ def _problem(seed, n, f, k, dtype=np.float32, lowcard=True):
     (2, 1, 1, 1, 256, np.float64),
     (1, 3, 2, 2, 8, np.float32),
     (700, 300, 1, 3, 5, np.float32),
+    (4000, 150, 1, 4, 256, np.float32),   # several feature groups, two features per lane
+    (6000, 64, 1, 5, 256, np.float32),    # one group, gradients embedded in the bin records
+    (2500, 18, 1, 4, 300, np.float64),    # two-byte bins with double features
 ])
 def test_build_tree_bit_exact(n, f, k, depth, s, dtype):
     import gpu_util as gu
@@ -87,6 +90,24 @@ def test_deep_tree_with_duplicates_and_small_nodes():
     gr, cr = gu.both(X, g, h, levels=True, max_depth=12, split_samples=512, seed=77)
     gu.assert_tree_parity(gr, cr, levels=True)
     assert (cr.feature != -1).sum() > 100
+
+
+def test_skewed_features_exercise_every_stage_of_the_bin_search():
+    """Heavy tails crowd most proposals into a few lookup cells, so the search runs through its
+    probe windows into the binary-search stage; a constant and a two-valued column sit beside them."""
+    import gpu_util as gu
+
+    rs = np.random.RandomState(11)
+    n, f = 20000, 24
+    X = np.exp(rs.randn(n, f) * 2.5).astype(np.float32)
+    X[:, 3] = 1.5
+    X[:, 4] = rs.randint(0, 2, n)
+    X[:, 5] = -np.exp(rs.randn(n) * 3.0)
+    X[::97, 6] = np.float32(3.0e38)
+    g = rs.randn(n, 1)
+    h = rs.rand(n, 1) + 0.5
+    gr, cr = gu.both(X, g, h, levels=True, max_depth=6, split_samples=256, seed=31)
+    gu.assert_tree_parity(gr, cr, levels=True)
 
 
 def test_tie_rule_on_gpu():
