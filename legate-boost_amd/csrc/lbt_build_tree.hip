@@ -324,6 +324,66 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// The same for several outputs per row: the (row, output) entries are walked in memory order
+// (the kernel above, launched once per output, would read every line K times). The grid stride
+// is a multiple of K, so a thread stays with one output and sums in registers; the outputs'
+// sums of a workgroup meet in LDS.
+constexpr int kQuantiseFlatMaxK = 2048;
+__global__ void __launch_bounds__(kThreads)
+  quantise_flat_kernel(const double* g, const double* h, int64_t n_rows, int K, int64_t row_offset, int64_t seed,
+                       const double* scales, int2* q_out, I64Pair* node_sums, unsigned long long* qstats)
+{
+  extern __shared__ unsigned long long s_sums[];  // [K] grad, [K] hess
+  __shared__ unsigned long long s_max;
+  for (int i = threadIdx.x; i < 2 * K; i += kThreads) s_sums[i] = 0;
+  if (threadIdx.x == 0) s_max = 0;
+  __syncthreads();
+  const double sg = scales[0], sh = scales[1];
+  const int64_t n       = n_rows * K;
+  const int64_t threads = static_cast<int64_t>(gridDim.x) * kThreads;
+  const int64_t stride  = threads / K * K;  // the launch makes sure that threads >= K
+  const int64_t first   = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  const int k           = static_cast<int>(first % K);
+  int64_t sum_g = 0, sum_h = 0;
+  unsigned long long mx = 0;
+  bool bad = false;
+  if (first < stride) {
+    for (int64_t e = first; e < n; e += stride) {
+      const int64_t row = e / K;
+      double grad = g[e], hess = h[e];
+      uint32_t x  = minstd_seed(static_cast<uint32_t>(
+        static_cast<uint64_t>(gpair_seed(seed, row + row_offset, static_cast<int64_t>(k)))));
+      double scaled_grad    = grad * sg;
+      double scaled_hess    = hess * sh;
+      double grad_remainder = scaled_grad - floor(scaled_grad);
+      double hess_remainder = scaled_hess - floor(scaled_hess);
+      x = minstd_next(x);
+      int64_t qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
+      x = minstd_next(x);
+      int64_t qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
+      bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
+      q_out[e] = make_int2(static_cast<int>(qg), static_cast<int>(qh));
+      unsigned long long ag = static_cast<unsigned long long>(qg < 0 ? -qg : qg);
+      unsigned long long ah = static_cast<unsigned long long>(qh < 0 ? -qh : qh);
+      mx = ag > mx ? ag : mx;
+      mx = ah > mx ? ah : mx;
+      sum_g += qg;
+      sum_h += qh;
+    }
+    atomicAdd(&s_sums[k], static_cast<unsigned long long>(sum_g));
+    atomicAdd(&s_sums[K + k], static_cast<unsigned long long>(sum_h));
+    atomicMax(&s_max, mx);
+  }
+  if (bad) atomicMax(&qstats[1], 1ULL);
+  __syncthreads();
+  for (int i = threadIdx.x; i < K; i += kThreads) {
+    const unsigned long long vg = s_sums[i], vh = s_sums[K + i];
+    if (vg != 0) atomic_add_i64(&node_sums[i].grad, static_cast<int64_t>(vg));
+    if (vh != 0) atomic_add_i64(&node_sums[i].hess, static_cast<int64_t>(vh));
+  }
+  if (threadIdx.x == 0) atomicMax(&qstats[0], s_max);
+}
+
 // build_tree.cu:1175-1185
 __global__ void root_leaf_kernel(double* leaf, const I64Pair* node_sums, int K,
                                  const double* scales, double l1, double l2)
@@ -1073,9 +1133,16 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       m = m2;
     }
     scales_kernel<<<1, 64, 0, stream>>>(L.part_a[cur], L.part_b[cur], L.scales, L.qstats);
-    dim3 grid(std::min<unsigned>(blocks(N, kThreads), 2048u), K);
-    quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(prm.seed),
-                                                   L.scales, L.qgh, L.node_sums, L.qstats);
+    if (K > 1 && K <= kQuantiseFlatMaxK) {
+      const unsigned gx = std::max<unsigned>(std::min<unsigned>(blocks(N * K, kThreads), 2048u),
+                                             blocks(K, kThreads));
+      quantise_flat_kernel<<<gx, kThreads, 2 * K * sizeof(unsigned long long), stream>>>(
+        g, h, N, K, row_offset, static_cast<int64_t>(prm.seed), L.scales, L.qgh, L.node_sums, L.qstats);
+    } else {
+      dim3 grid(std::min<unsigned>(blocks(N, kThreads), 2048u), K);
+      quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(prm.seed),
+                                                     L.scales, L.qgh, L.node_sums, L.qstats);
+    }
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization);
   }
