@@ -207,7 +207,8 @@ def bench_training(args):
     for d, lv in enumerate(prof["levels"]):
         # the library's own figure prices a feature value at its cached width; what is left of it
         # after the row terms are the histograms written
-        written = max(0.0, lv["bytes"] - lv["built_instances"] * (f * bin_bytes + k * 8.0 + 8.0))
+        own_extra = n * f * bin_bytes * steps if (d == 0 and depth >= 2) else 0.0  # feature-major copy, root launch
+        written = max(0.0, lv["bytes"] - own_extra - lv["built_instances"] * (f * bin_bytes + k * 8.0 + 8.0))
         ref_bytes = lv["built_instances"] * (f * elem + k * 8.0) + lv["instances"] * 8.0 + written
         stage_bytes += ref_bytes
         levels.append({"level": d, "ms": lv["ms"] / steps, "built_rows": lv["built_instances"] / steps,

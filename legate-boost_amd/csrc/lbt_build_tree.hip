@@ -655,48 +655,7 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
-// Feature-major copy of the bin cache: out[f][row]. One workgroup turns 128
-// rows of one group through LDS, 64 features at a time, so that both sides move
-// whole 4-byte words. `base`/`stride` locate a feature's bins in the cache.
-constexpr int kTransRows = 128;
-constexpr int kTransFeat = kTransposeFeatures;
-template <typename BinT>
-__global__ void __launch_bounds__(kThreads)
-  transpose_bins_kernel(const BinT* cache, const int32_t* groups, const int64_t* base, const int32_t* stride,
-                        int64_t n_rows, int64_t out_stride, BinT* out)
-{
-  constexpr int per_w  = 4 / sizeof(BinT);                  // elements per 32-bit word
-  constexpr int lpitch = kTransFeat / per_w + 1;            // odd word pitch spreads a column over the banks
-  __shared__ uint32_t s_words[kTransRows * lpitch];
-  const int64_t r0 = blockIdx.x * static_cast<int64_t>(kTransRows);
-  const int f0 = groups[blockIdx.y], f1 = groups[blockIdx.y + 1];
-  const int pitch = stride[f0];
-  for (int fa = f0; fa < f1; fa += kTransFeat) {
-    const int fb      = min(f1, fa + kTransFeat);
-    const int n_words = (fb - fa + per_w - 1) / per_w;
-    const BinT* src   = cache + base[fa];  // 4-byte aligned: group starts and fa - f0 are multiples of 4 bytes
-    __syncthreads();
-    for (int i = threadIdx.x; i < kTransRows * n_words; i += kThreads) {
-      int r = i / n_words, wi = i % n_words;
-      uint32_t v = 0;
-      if (r0 + r < n_rows) v = reinterpret_cast<const uint32_t*>(src + (r0 + r) * pitch)[wi];
-      s_words[r * lpitch + wi] = v;
-    }
-    __syncthreads();
-    const BinT* s_el       = reinterpret_cast<const BinT*>(s_words);
-    constexpr int row_sets = kTransRows / per_w;  // output words per feature
-    for (int i = threadIdx.x; i < (fb - fa) * row_sets; i += kThreads) {
-      int f = fa + i / row_sets, rs = i % row_sets;
-      uint32_t word = 0;
-#pragma unroll
-      for (int j = 0; j < per_w; j++) {
-        uint32_t b = s_el[static_cast<size_t>(rs * per_w + j) * lpitch * per_w + (f - fa)];
-        word |= b << (8 * sizeof(BinT) * j);
-      }
-      reinterpret_cast<uint32_t*>(out + f * out_stride + r0)[rs] = word;
-    }
-  }
-}
+constexpr int kTransRows = 128;  // the feature-major bins are padded to whole groups of this many rows
 
 // pass 1 when the feature-major bins exist: x <= proposals[b] holds exactly when the
 // row's bin (first proposal that is not below x) is <= b, so the split feature's bin
@@ -1181,6 +1140,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.bin_stride = L.bin_stride;
   hs.bin_tail   = L.bin_tail;
   hs.rec        = L.rec;
+  // feature-major bins for the position updates of levels 0 .. max_depth-2 (and the final leaves)
+  hs.bins_t        = L.binned != nullptr ? L.bins_t : nullptr;
+  hs.bins_t_stride = L.bins_t_stride;
   hs.meta       = L.meta;
   LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
 
@@ -1262,19 +1224,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
                                                        n_chunks, L.partial, leaf, feature, split, gain, L.row_pointers,
                                                        L.split_bin);
       }
-    }
-    if (depth == 0 && use_bins_t) {
-      // feature-major copy of the bins the root pass has just cached
-      ProfScope ps(LBT_PROF_POSITIONS, stream);
-      dim3 grid(blocks(N, kTransRows), hs.n_groups);
-      if (hs.bin_bytes == 1)
-        transpose_bins_kernel<uint8_t><<<grid, kThreads, 0, stream>>>(
-          static_cast<const uint8_t*>(hs.binned), hs.groups, hs.bin_base, hs.bin_stride, N, L.bins_t_stride,
-          static_cast<uint8_t*>(L.bins_t));
-      else
-        transpose_bins_kernel<uint16_t><<<grid, kThreads, 0, stream>>>(
-          static_cast<const uint16_t*>(hs.binned), hs.groups, hs.bin_base, hs.bin_stride, N, L.bins_t_stride,
-          static_cast<uint16_t*>(L.bins_t));
     }
     if (depth < max_depth - 1) {
       ProfScope ps(LBT_PROF_POSITIONS, stream, static_cast<double>(N) * (8 + 8 + 2 + 64));
@@ -1368,6 +1317,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       double per_value = cached ? hs.bin_bytes : static_cast<double>(sizeof(T));
       double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * per_value + K * 8.0 + 8.0) +
                   static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
+      // the root launch also writes the feature-major copy of the bins
+      if (d == 0 && hs.bins_t != nullptr) by += static_cast<double>(N) * F * hs.bin_bytes;
       acc.level_bytes[d] += by;
       acc.level_instances[d] += static_cast<double>(h_levels[d].instances);
       acc.level_built_instances[d] += static_cast<double>(h_levels[d].built_instances);

@@ -777,15 +777,33 @@ struct BinnedArgs {
   HistView hist;
 };
 
+// 4 x 4 byte transpose: input word r is row r and its byte b is feature b; output word b holds
+// feature b of rows 0..3.
+__device__ __forceinline__ void turn_bytes(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t (&out)[4])
+{
+  const uint32_t a = __builtin_amdgcn_perm(w1, w0, 0x05010400u);
+  const uint32_t b = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
+  const uint32_t c = __builtin_amdgcn_perm(w3, w2, 0x05010400u);
+  const uint32_t d = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
+  out[0]           = __builtin_amdgcn_perm(c, a, 0x05040100u);
+  out[1]           = __builtin_amdgcn_perm(c, a, 0x07060302u);
+  out[2]           = __builtin_amdgcn_perm(d, b, 0x05040100u);
+  out[3]           = __builtin_amdgcn_perm(d, b, 0x07060302u);
+}
+
 // kEmbed: the records carry the packed (grad, hess) of their row (single-output trees);
 // otherwise the pair of (row, output) is gathered from qgh.
-template <typename BinT, int BV, bool kEmbed>
+// kRoot: the launch for the root, whose rows are still in their original order. A lane then
+// takes four consecutive rows per tile and, besides accumulating, stores their bins feature by
+// feature into bins_t ([feature][row]), which the position updates read: the feature-major copy
+// costs no second pass over the cache.
+template <typename BinT, int BV, bool kEmbed, bool kRoot>
 __global__ void __launch_bounds__(kHistThreads)
   binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
-                          const int2* __restrict__ qgh)
+                          const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride)
 {
   using Word = typename BinVec<BinT, BV>::type;
-  constexpr int kRows = BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll;  // rows per lane and tile
+  constexpr int kRows = kRoot ? 4 : (BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll);  // rows per lane and tile
   extern __shared__ unsigned char smem_raw[];
   const TileWalk& w = a.w;
   const int xcd   = blockIdx.x & 7;
@@ -829,9 +847,12 @@ __global__ void __launch_bounds__(kHistThreads)
     unsigned valid = 0;
 #pragma unroll
     for (int u = 0; u < kRows; u++) {
-      const int rr  = t.r0 + rsub + u * w.rpp;
+      const int rr  = kRoot ? t.r0 + kRows * rsub + u : t.r0 + rsub + u * w.rpp;
       const bool ok = active && rr < t.r1;
-      row[u]        = positions[ok ? rr : t.r0].y;
+      if constexpr (kRoot)
+        row[u] = ok ? rr : t.r0;  // the order is still the identity: sorted index == row
+      else
+        row[u] = positions[ok ? rr : t.r0].y;
       valid |= ok ? (1u << u) : 0u;
     }
     return valid;
@@ -893,6 +914,42 @@ __global__ void __launch_bounds__(kHistThreads)
       for (int u = 0; u < kRows; u++) {
         b_c[u].z = strip ? 0u : b_c[u].z;
         b_c[u].w = strip ? 0u : b_c[u].w;
+      }
+    }
+    if constexpr (kRoot) {
+      // feature-major copy (one output's workgroups do it); rows past the end of the tile hold
+      // the bins of the tile's first row, and bins_t is padded to whole groups of rows
+      if (k == 0 && (valid_c & 1u)) {
+        const int64_t row0 = row_c[0];
+        if constexpr (BV == 16) {
+          BinT* dst = bins_t + static_cast<int64_t>(f0 + fl) * bins_t_stride + row0;
+          auto put  = [&](int i, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+            uint32_t o[4];
+            turn_bytes(w0, w1, w2, w3, o);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              if (fl + 4 * i + j < gs) *reinterpret_cast<uint32_t*>(dst) = o[j];
+              dst += bins_t_stride;
+            }
+          };
+          put(0, b_c[0].x, b_c[1].x, b_c[2].x, b_c[3].x);
+          put(1, b_c[0].y, b_c[1].y, b_c[2].y, b_c[3].y);
+          put(2, b_c[0].z, b_c[1].z, b_c[2].z, b_c[3].z);
+          put(3, b_c[0].w, b_c[1].w, b_c[2].w, b_c[3].w);
+        } else {
+          // four two-byte bins per row
+          const uint32_t lo[4] = {b_c[0].x, b_c[1].x, b_c[2].x, b_c[3].x};
+          const uint32_t hi[4] = {b_c[0].y, b_c[1].y, b_c[2].y, b_c[3].y};
+          uint2 o[4];
+          o[0] = make_uint2((lo[0] & 0xffffu) | (lo[1] << 16), (lo[2] & 0xffffu) | (lo[3] << 16));
+          o[1] = make_uint2((lo[0] >> 16) | (lo[1] & 0xffff0000u), (lo[2] >> 16) | (lo[3] & 0xffff0000u));
+          o[2] = make_uint2((hi[0] & 0xffffu) | (hi[1] << 16), (hi[2] & 0xffffu) | (hi[3] << 16));
+          o[3] = make_uint2((hi[0] >> 16) | (hi[1] & 0xffff0000u), (hi[2] >> 16) | (hi[3] & 0xffff0000u));
+#pragma unroll
+          for (int v = 0; v < 4; v++)
+            if (fl + v < gs)
+              *reinterpret_cast<uint2*>(bins_t + static_cast<int64_t>(f0 + fl + v) * bins_t_stride + row0) = o[v];
+        }
       }
     }
     if (!direct) {
@@ -992,17 +1049,25 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
   return launch_bin_rows<T, VEC, uint16_t>(stream, hs, a, b, grid);
 }
 
-template <typename BinT, int BV, bool kEmbed>
-int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
+template <typename BinT, int BV, bool kEmbed, bool kRoot>
+int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
 {
   static bool attr_set = false;
   if (!attr_set) {
-    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV, kEmbed>));
+    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>));
     attr_set = true;
   }
-  binned_histogram_kernel<BinT, BV, kEmbed><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
-    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh);
+  binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
+    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
+    static_cast<BinT*>(hs.bins_t), hs.bins_t_stride);
   return LBT_OK;
+}
+template <typename BinT, int BV, bool kEmbed>
+int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
+                  bool root)
+{
+  if (root) return launch_binned_as<BinT, BV, kEmbed, true>(stream, hs, a, b, grid);
+  return launch_binned_as<BinT, BV, kEmbed, false>(stream, hs, a, b, grid);
 }
 
 // As many resident workgroups as the LDS allows per CU; row-tile ranges come in multiples
@@ -1072,10 +1137,12 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     }
     LBT_TRY(rc);
   }
+  // the root launch on cached bins also writes the feature-major copy (four rows per lane and tile)
+  const bool root = use_cache && depth == 0 && hs.bins_t != nullptr;
   TileWalk w;
   unsigned grid = 0;
   LBT_TRY(fill_walk(w, b, n_cu, hs.n_groups, use_cache ? hs.brpp : hs.rpp,
-                    use_cache ? (hs.bvec == 16 ? kBinnedUnroll / 2 : kBinnedUnroll) : kUnroll,
+                    use_cache ? (root ? 4 : (hs.bvec == 16 ? kBinnedUnroll / 2 : kBinnedUnroll)) : kUnroll,
                     use_cache ? hs.blds_bytes : hs.lds_bytes, &grid));
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
@@ -1097,10 +1164,10 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     a.groups       = hs.groups;
     a.hist         = b.hist;
     if (hs.bin_bytes == 1)
-      return hs.embed ? launch_binned<uint8_t, 16, true>(stream, hs, a, b, grid)
-                      : launch_binned<uint8_t, 16, false>(stream, hs, a, b, grid);
-    return hs.embed ? launch_binned<uint16_t, 4, true>(stream, hs, a, b, grid)
-                    : launch_binned<uint16_t, 4, false>(stream, hs, a, b, grid);
+      return hs.embed ? launch_binned<uint8_t, 16, true>(stream, hs, a, b, grid, root)
+                      : launch_binned<uint8_t, 16, false>(stream, hs, a, b, grid, root);
+    return hs.embed ? launch_binned<uint16_t, 4, true>(stream, hs, a, b, grid, root)
+                    : launch_binned<uint16_t, 4, false>(stream, hs, a, b, grid, root);
   }
   HistArgs<T> a;
   a.w            = w;

@@ -302,12 +302,15 @@ struct HistSetup {
   int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
   int32_t* bin_stride  = nullptr;  // [n_features] elements between consecutive rows
   int32_t* bin_tail    = nullptr;  // [n_features] g + 1 for the last feature of histogram group g, else 0
+  // feature-major copy of the bins, [feature][row], written by the root histogram launch for the
+  // position updates (null: not wanted)
+  void* bins_t           = nullptr;
+  int64_t bins_t_stride  = 0;      // elements between consecutive features (multiple of 128)
   int rpp              = 0;        // rows per workgroup pass, search / binning kernel
   int brpp             = 0;        // rows per workgroup pass, histogram kernel on cached bins
 };
 
 constexpr int kMaxCells = 2048;
-constexpr int kTransposeFeatures = 64;  // features the bin transpose stages at a time
 constexpr int kHistThreads       = 1024;
 // LDS a histogram-stage workgroup may fill; 4 KB of the 160 KB stay free for the tile window
 constexpr size_t kLdsBudget = 160 * 1024 - 512 - 4096;
