@@ -635,43 +635,49 @@ __global__ void __launch_bounds__(kHistThreads)
     tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
     tz_words         = ((ri.bins_end | ri.zero_end) & 3) == 0;
   }
-  const T* const x_base = X + fb;
   const int64_t r_begin = a.n_rows * chunk / a.n_chunks;
   const int64_t r_end   = a.n_rows * (chunk + 1) / a.n_chunks;
+  // Inside the chunk rows are numbered from 0 and addressed by 32-bit byte offsets (the host
+  // keeps a chunk's rows times the widest row below 2^31 bytes), which advance by a uniform
+  // step from pass to pass instead of being multiplied out per row.
+  const int n_local                  = static_cast<int>(r_end - r_begin);
+  const unsigned char* const x_chunk = reinterpret_cast<const unsigned char*>(X + r_begin * a.F + fb);
+  const int2* const q_chunk          = qgh + r_begin;
+  unsigned char* const b_chunk       = reinterpret_cast<unsigned char*>(bin_base + r_begin * pitch);
+  const uint32_t row_bytes = static_cast<uint32_t>(a.F) * sizeof(T);
+  const uint32_t rec_bytes = static_cast<uint32_t>(pitch) * sizeof(BinT);
+  const uint32_t x_step    = static_cast<uint32_t>(a.rpp) * row_bytes;  // from one row of a pass to the next
+  const uint32_t b_step    = static_cast<uint32_t>(a.rpp) * rec_bytes;
+  const uint32_t x_last    = n_local > 0 ? static_cast<uint32_t>(n_local - 1) * row_bytes : 0u;
+  const int pass_rows      = a.rpp * kUnroll;
   __syncthreads();
 
-  // pass p covers rows r_begin + (p * kUnroll + u) * rpp + rsub; the values of the next pass
-  // are requested before the current one is searched
-  auto load_pass = [&](int64_t first, Vec (&xv)[kUnroll]) {
+  // pass p covers local rows (p * kUnroll + u) * rpp + rsub; the values of the next pass are
+  // requested before the current one is searched. Rows past the chunk's end (and the lanes
+  // without a row) read its last row instead.
+  auto load_pass = [&](int first, Vec (&xv)[kUnroll]) {
+    const uint32_t off0 = static_cast<uint32_t>(first + rsub) * row_bytes;
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
-      r         = (active && r < r_end) ? r : r_begin;
-      const T* xp = x_base + r * a.F;
+      const uint32_t off = min(off0 + u * x_step, x_last);
       if constexpr (VEC == 1)
-        xv[u] = *xp;
+        xv[u] = *reinterpret_cast<const T*>(x_chunk + off);
       else
-        xv[u] = *reinterpret_cast<const Vec*>(xp);
+        xv[u] = *reinterpret_cast<const Vec*>(x_chunk + off);
     }
   };
-  const int64_t pass_rows = static_cast<int64_t>(a.rpp) * kUnroll;
-  Vec x_c[kUnroll], x_n[kUnroll];
-  int2 q_c[kUnroll];
-  if (r_begin < r_end) load_pass(r_begin, x_c);
-  for (int64_t first = r_begin; first < r_end; first += pass_rows) {
-    if (first + pass_rows < r_end) load_pass(first + pass_rows, x_n);
+  auto search_pass = [&](int first, const Vec (&x_c)[kUnroll]) {
     // the few lanes that copy gradient pairs fetch them now; the search below hides the latency
+    int2 q_c[kUnroll];
     if (tq >= 0) {
 #pragma unroll
-      for (int u = 0; u < kUnroll; u++) {
-        const int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
-        q_c[u]          = qgh[(active && r < r_end) ? r : r_begin];
-      }
+      for (int u = 0; u < kUnroll; u++) q_c[u] = q_chunk[min(first + u * a.rpp + rsub, n_local - 1)];
     }
+    const uint32_t b_off0 = static_cast<uint32_t>(first + rsub) * rec_bytes;
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
-      const int64_t r = first + static_cast<int64_t>(u) * a.rpp + rsub;
-      if (active && r < r_end) {
+      const int r = first + u * a.rpp + rsub;
+      if (active && r < n_local) {
         T xs[VEC];
         if constexpr (VEC == 1) {
           xs[0] = x_c[u];
@@ -711,7 +717,8 @@ __global__ void __launch_bounds__(kHistThreads)
           }
           rel[v] = static_cast<BinT>(bn[v] + cnt[v] - c_prop[v]);
         }
-        BinT* bp = bin_base + r * pitch;
+        unsigned char* tail = b_chunk + (b_off0 + u * b_step);
+        BinT* bp            = reinterpret_cast<BinT*>(tail);
         if constexpr (VEC == 4 && sizeof(BinT) == 1) {
           *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
                                              (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
@@ -720,7 +727,6 @@ __global__ void __launch_bounds__(kHistThreads)
           for (int v = 0; v < VEC; v++) bp[v] = rel[v];
         }
         if (tg > 0) {
-          unsigned char* tail = reinterpret_cast<unsigned char*>(bp);
           if (tz_words) {
             for (int i = tz_from; i < tz_to; i += 4) *reinterpret_cast<uint32_t*>(tail + i) = 0u;
           } else {
@@ -730,6 +736,12 @@ __global__ void __launch_bounds__(kHistThreads)
         }
       }
     }
+  };
+  Vec x_c[kUnroll], x_n[kUnroll];
+  if (n_local > 0) load_pass(0, x_c);
+  for (int first = 0; first < n_local; first += pass_rows) {
+    if (first + pass_rows < n_local) load_pass(first + pass_rows, x_n);
+    search_pass(first, x_c);
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) x_c[u] = x_n[u];
   }
@@ -1125,6 +1137,9 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     const int per_cu = hs.lds_bytes * 2 <= 160 * 1024 ? 2 : 1;
     int64_t per_xcd  = std::max<int64_t>(1, (per_cu * n_cu / 8) / hs.n_sgroups);
     per_xcd          = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (b.n_rows / (hs.rpp * kUnroll) + 7) / 8));
+    // the kernel addresses a chunk's rows with 32-bit byte offsets
+    const int64_t widest = std::max<int64_t>(static_cast<int64_t>(b.F) * sizeof(T), hs.max_rec_stride);
+    while ((b.n_rows / (per_xcd * 8) + 2) * widest >= (int64_t(1) << 31)) per_xcd *= 2;
     a.n_chunks       = static_cast<int>(per_xcd * 8);
     const unsigned grid = static_cast<unsigned>(per_xcd * 8 * hs.n_sgroups);
     int rc = LBT_OK;
@@ -1354,6 +1369,7 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       }
       const int used = std::max(chunk_end, hs.embed ? ri.q_off + 8 : 0);
       ri.stride      = (used + 31) / 32 * 32;
+      hs.max_rec_stride = std::max<int64_t>(hs.max_rec_stride, ri.stride);
       ri.base        = at;
       for (int f = groups[g]; f < groups[g + 1]; f++) {
         base[f]   = at / hs.bin_bytes + (f - groups[g]);

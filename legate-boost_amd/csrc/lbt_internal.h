@@ -299,6 +299,7 @@ struct HistSetup {
   bool embed           = false;    // records carry the row's (grad, hess)
   size_t blds_bytes    = 0;        // LDS of the histogram kernel (packed sub-histogram only)
   RecInfo* rec         = nullptr;  // [n_groups]
+  int64_t max_rec_stride = 0;      // widest record, bytes
   int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
   int32_t* bin_stride  = nullptr;  // [n_features] elements between consecutive rows
   int32_t* bin_tail    = nullptr;  // [n_features] g + 1 for the last feature of histogram group g, else 0
