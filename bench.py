@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the tree-learner path on one MI355X.
 
-Default workload: BASELINE config 2 -- LBRegressor squared error,
+Default workload (configuration 2 of the benchmark plan): LBRegressor squared error,
 Tree(max_depth=8, split_samples=256), X 10,000,000 x 100 f32. One step is one
 boosting round: gradient step, BuildTreeTask, PredictTask of the new tree and
 the prediction update, all with inputs resident in HBM.

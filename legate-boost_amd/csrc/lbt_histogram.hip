@@ -1012,22 +1012,11 @@ __global__ void __launch_bounds__(kHistThreads)
   if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
 }
 
-template <typename KernelT>
-int allow_large_lds(KernelT kernel)
-{
-  LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              static_cast<int>(kLdsBudget)));
-  return LBT_OK;
-}
-
 template <typename T, int VEC, bool kIdentityRows>
 int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, const HistBatch& b, unsigned grid)
 {
-  static bool attr_set = false;
-  if (!attr_set) {
-    LBT_TRY(allow_large_lds(histogram_kernel<T, VEC, kIdentityRows>));
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  LBT_TRY(allow_dynamic_lds(histogram_kernel<T, VEC, kIdentityRows>, kLdsBudget, attr_set));
   histogram_kernel<T, VEC, kIdentityRows><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
     a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const T*>(b.X), b.qgh);
   return LBT_OK;
@@ -1044,11 +1033,8 @@ int launch_search_rows(hipStream_t stream, const HistSetup& hs, const HistArgs<T
 template <typename T, int VEC, typename BinT>
 int launch_bin_rows(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
 {
-  static bool attr_set = false;
-  if (!attr_set) {
-    LBT_TRY(allow_large_lds(bin_rows_kernel<T, VEC, BinT>));
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  LBT_TRY(allow_dynamic_lds(bin_rows_kernel<T, VEC, BinT>, kLdsBudget, attr_set));
   bin_rows_kernel<T, VEC, BinT><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a, static_cast<const T*>(b.X), b.qgh,
                                                                             static_cast<BinT*>(hs.binned));
   return LBT_OK;
@@ -1064,11 +1050,8 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
 template <typename BinT, int BV, bool kEmbed, bool kRoot>
 int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
 {
-  static bool attr_set = false;
-  if (!attr_set) {
-    LBT_TRY(allow_large_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>));
-    attr_set = true;
-  }
+  static bool attr_set[kMaxDevices] = {};
+  LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride);

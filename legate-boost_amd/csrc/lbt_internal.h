@@ -227,6 +227,22 @@ __device__ inline bool compute_histogram_bin(int node, const I64Pair* node_sums,
   return histogram_node == node;
 }
 
+// Lets `kernel` use up to `bytes` of dynamic LDS. The attribute belongs to the device the
+// function is loaded on, so it is set once per device; `done` is the caller's per-kernel record
+// (one flag per device ordinal). Setting it twice from two threads is harmless.
+constexpr int kMaxDevices = 64;
+template <typename KernelT>
+int allow_dynamic_lds(KernelT kernel, size_t bytes, bool (&done)[kMaxDevices])
+{
+  int device = 0;
+  LBT_HIP(hipGetDevice(&device));
+  if (device >= 0 && device < kMaxDevices && done[device]) return LBT_OK;
+  LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              static_cast<int>(bytes)));
+  if (device >= 0 && device < kMaxDevices) done[device] = true;
+  return LBT_OK;
+}
+
 inline int ceil_div(int64_t a, int64_t b) { return static_cast<int>((a + b - 1) / b); }
 
 __device__ inline void atomic_add_i64(int64_t* p, int64_t v)

@@ -512,14 +512,9 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
     for (int i = 0; i < n; i++) tb.b[i] = binfo[first + i];
     write_batches_kernel<<<1, kPackBatches, 0, stream>>>(tb, first, n, batches);
   }
-  static bool attr_set = false;
-  if (!attr_set) {
-    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(predict_tile_kernel<T, true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kTileLds)));
-    LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(predict_tile_kernel<T, false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kTileLds)));
-    attr_set = true;
-  }
+  static bool attr_single[kMaxDevices] = {}, attr_multi[kMaxDevices] = {};
+  LBT_TRY(allow_dynamic_lds(predict_tile_kernel<T, true>, kTileLds, attr_single));
+  LBT_TRY(allow_dynamic_lds(predict_tile_kernel<T, false>, kTileLds, attr_multi));
   const unsigned tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
   if (K == 1)
     predict_tile_kernel<T, true><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,

@@ -131,7 +131,7 @@ def test_tie_rule_on_gpu():
 
 
 def test_config1_boosting_rounds_match_oracle_round_by_round():
-    """BASELINE config 1: 100000x32, squared error, depth 6, 10 rounds, lr 0.1.
+    """Benchmark configuration 1: 100000x32, squared error, depth 6, 10 rounds, lr 0.1.
     Each round's task inputs (X, g, h, seed) go to both implementations."""
     import gpu_util as gu
     import oracle_lib as orc
