@@ -230,7 +230,7 @@ __global__ void __launch_bounds__(kThreads)
   sb[threadIdx.x] = xb;
   __syncthreads();
   for (int stride = kThreads / 2; stride >= 1; stride >>= 1) {
-    if (threadIdx.x < stride) {
+    if (static_cast<int>(threadIdx.x) < stride) {
       sa[threadIdx.x] += sa[threadIdx.x + stride];
       sb[threadIdx.x] += sb[threadIdx.x + stride];
     }

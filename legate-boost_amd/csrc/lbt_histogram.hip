@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(kPlanThreads)
     s_scan[threadIdx.x] = tiles;
     __syncthreads();
     for (int off = 1; off < kPlanThreads; off <<= 1) {
-      int v = threadIdx.x >= off ? s_scan[threadIdx.x - off] : 0;
+      int v = static_cast<int>(threadIdx.x) >= off ? s_scan[threadIdx.x - off] : 0;
       __syncthreads();
       s_scan[threadIdx.x] += v;
       __syncthreads();
