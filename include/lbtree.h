@@ -119,7 +119,7 @@ size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t
  *   tree_nodes          HOST array: number of nodes of each tree
  *   out                 device double [n_rows][n_outputs]; overwritten
  *   workspace           device scratch of at least lbt_predict_workspace_bytes(...), or
- *                       NULL. With it, rows are staged in LDS in tiles of 256 and walked
+ *                       NULL. With it, rows are staged in LDS in tiles of 64 to 256 and walked
  *                       through the packed ensemble batch by batch; without it (or when a
  *                       row tile or a tree does not fit the LDS, or n_outputs > 8) every
  *                       node step reads the trees' own arrays. The sums are the same: a

@@ -99,10 +99,11 @@ int predict_impl(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
 // X's type, feature, and the index of the right child. A leaf is packed as a node that always
 // steps to itself (threshold NaN, "right child" = itself), so a walk is a fixed number of
 // identical steps with no test for leaves.
-// A workgroup then owns a tile of 256 rows: it stages the rows in LDS once and walks them
-// through all trees, a batch of up to 20 trees at a time that is copied into LDS too, so a node
-// step costs two LDS reads and no trip to the L2. Four lanes share a row and take every fourth
-// tree of the batch, five trees each, interleaved for latency. The nodes of the next batch are
+// A workgroup then owns a tile of rows (256, or fewer for wide matrices): it stages the rows in
+// LDS once and walks them through all trees, a batch of trees at a time that is copied into LDS
+// too, so a node step costs two LDS reads and no trip to the L2. Four lanes (8 or 16 for wide
+// matrices) share a row and take every fourth tree of the batch, a few trees each, interleaved
+// for latency. The nodes of the next batch are
 // fetched into registers while the current one is walked, and the leaf values of a batch are
 // fetched (from a packed copy) while the next one is walked. They are added in tree order, so a row's sum is formed
 // exactly as the per-tree launches of the reference form it.
@@ -138,10 +139,15 @@ struct alignas(8) BatchInfo {
 constexpr int kPackTrees    = 64;  // trees packed per launch (descriptors passed by value)
 constexpr int kPackBatches  = 128; // batch descriptors written per launch
 constexpr int kTileThreads  = 1024;
-constexpr int kTileRows     = 256;
-constexpr int kRowLanes     = 4;
-constexpr int kLaneTrees    = 5;
-constexpr int kBatchTrees   = kRowLanes * kLaneTrees;
+// L lanes share a row; a workgroup then covers 1024 / L rows, and a batch holds L * kLaneTrees
+// trees. Wide feature matrices take more lanes per row, so that the row tile still fits the LDS.
+template <int L>
+struct TileShape {
+  static constexpr int kRowLanes   = L;
+  static constexpr int kRows       = kTileThreads / L;
+  static constexpr int kLaneTrees  = L == 4 ? 5 : (L == 8 ? 3 : 2);
+  static constexpr int kBatchTrees = kRowLanes * kLaneTrees;
+};
 constexpr int kTileMaxK     = 8;
 constexpr size_t kTileLds   = 160 * 1024 - 2048;  // dynamic LDS of the tile kernel
 constexpr int kCopyWords    = 6;  // 16-byte words a thread moves per batch: 6 * 1024 * 16 B >= any batch
@@ -214,41 +220,46 @@ __global__ void write_batches_kernel(BatchTable t, int first, int n, BatchInfo* 
   if (i < n) out[first + i] = t.b[i];
 }
 
-template <int kLane>
-__device__ inline int quad_broadcast(int v)
+// Every lane of a group of L lanes reads lane kLane of its group (groups of four through a
+// quad permute, wider ones through a lane-indexed shuffle).
+template <int L, int kLane>
+__device__ inline int group_broadcast(int v)
 {
-  // every lane of a group of four reads lane kLane of its group
-  return __builtin_amdgcn_mov_dpp(v, kLane * 0x55, 0xf, 0xf, false);
+  if constexpr (L == 4)
+    return __builtin_amdgcn_mov_dpp(v, kLane * 0x55, 0xf, 0xf, false);
+  else
+    return __shfl(v, (static_cast<int>(threadIdx.x) & 63 & ~(L - 1)) | kLane, 64);
 }
-template <int kLane>
-__device__ inline double quad_broadcast(double v)
+template <int L, int kLane>
+__device__ inline double group_broadcast(double v)
 {
   const long long bits = __double_as_longlong(v);
-  const int lo = quad_broadcast<kLane>(static_cast<int>(bits));
-  const int hi = quad_broadcast<kLane>(static_cast<int>(bits >> 32));
+  const int lo = group_broadcast<L, kLane>(static_cast<int>(bits));
+  const int hi = group_broadcast<L, kLane>(static_cast<int>(bits >> 32));
   return __longlong_as_double((static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
 }
-// value of tree jj of a batch, held by lane jj % 4 of the row's four lanes in slot jj / 4
-template <int jj, typename V>
-__device__ inline V from_owner(const V (&slots)[5])
+// value of tree jj of a batch, held by lane jj % L of the row's lanes in slot jj / L
+template <typename S, int jj, typename V>
+__device__ inline V from_owner(const V (&slots)[S::kLaneTrees])
 {
-  return quad_broadcast<jj & 3>(slots[jj >> 2]);
+  return group_broadcast<S::kRowLanes, jj % S::kRowLanes>(slots[jj / S::kRowLanes]);
 }
 
 // What is fetched one batch ahead: the nodes as 16-byte words and where this lane's trees start
 // inside the batch.
 typedef unsigned int Word16 __attribute__((ext_vector_type(4)));  // plain vector: stays in registers
+template <typename S>
 struct Prefetched {
   Word16 words[kCopyWords];
-  int base[kLaneTrees];
+  int base[S::kLaneTrees];
 };
 
-template <typename T>
-__device__ __forceinline__ Prefetched fetch_batch(const BatchInfo& bi, const PackedNode<T>* __restrict__ nodes,
+template <typename T, typename S>
+__device__ __forceinline__ Prefetched<S> fetch_batch(const BatchInfo& bi, const PackedNode<T>* __restrict__ nodes,
                                                   const PackedTree* __restrict__ desc, int q)
 {
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
-  Prefetched pf;
+  Prefetched<S> pf;
   // the packed array is 16-byte aligned and batches start on 16-byte boundaries (see predict_tiled)
   const Word16* src = reinterpret_cast<const Word16*>(nodes + bi.node_off);
   const int n16     = (bi.total + kNodesPerWord - 1) / kNodesPerWord;
@@ -258,55 +269,58 @@ __device__ __forceinline__ Prefetched fetch_batch(const BatchInfo& bi, const Pac
     pf.words[c] = src[i < n16 ? i : 0];
   }
 #pragma unroll
-  for (int j = 0; j < kLaneTrees; j++) {
-    const int jj = q + kRowLanes * j;
+  for (int j = 0; j < S::kLaneTrees; j++) {
+    const int jj = q + S::kRowLanes * j;
     pf.base[j]   = desc[bi.first + (jj < bi.count ? jj : 0)].rel_off;  // lanes without a tree walk tree 0 again
   }
   return pf;
 }
 
-template <int jj>
-__device__ __forceinline__ void add_in_order_from(double& acc, const double (&val)[kLaneTrees], int cnt)
+template <typename S, int jj>
+__device__ __forceinline__ void add_in_order_from(double& acc, const double (&val)[S::kLaneTrees], int cnt)
 {
-  if constexpr (jj < kBatchTrees) {
-    const double v = from_owner<jj>(val);
+  if constexpr (jj < S::kBatchTrees) {
+    const double v = from_owner<S, jj>(val);
     if (jj < cnt) acc += v;
-    add_in_order_from<jj + 1>(acc, val, cnt);
+    add_in_order_from<S, jj + 1>(acc, val, cnt);
   }
 }
-__device__ __forceinline__ void add_in_order(double& acc, const double (&val)[kLaneTrees], int cnt)
+template <typename S>
+__device__ __forceinline__ void add_in_order(double& acc, const double (&val)[S::kLaneTrees], int cnt)
 {
-  add_in_order_from<0>(acc, val, cnt);
+  add_in_order_from<S, 0>(acc, val, cnt);
 }
-template <int kAcc, int jj>
-__device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[kLaneTrees], int cnt,
+template <typename S, int kAcc, int jj>
+__device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
                                                 const double* __restrict__ batch_leaves, int K)
 {
-  if constexpr (jj < kBatchTrees) {
-    const int p = from_owner<jj>(at);
+  if constexpr (jj < S::kBatchTrees) {
+    const int p = from_owner<S, jj>(at);
     if (jj < cnt) {
       const double* lf = batch_leaves + static_cast<int64_t>(p) * K;
 #pragma unroll
       for (int k = 0; k < kAcc; k++)
         if (k < K) acc[k] += lf[k];
     }
-    add_leaves_from<kAcc, jj + 1>(acc, at, cnt, batch_leaves, K);
+    add_leaves_from<S, kAcc, jj + 1>(acc, at, cnt, batch_leaves, K);
   }
 }
-template <int kAcc>
-__device__ __forceinline__ void add_leaves_in_order(double (&acc)[kAcc], const int (&at)[kLaneTrees], int cnt,
+template <typename S, int kAcc>
+__device__ __forceinline__ void add_leaves_in_order(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
                                                     const double* __restrict__ batch_leaves, int K)
 {
-  add_leaves_from<kAcc, 0>(acc, at, cnt, batch_leaves, K);
+  add_leaves_from<S, kAcc, 0>(acc, at, cnt, batch_leaves, K);
 }
 
-template <typename T, bool kSingle>
+template <typename T, bool kSingle, int L>
 __global__ void __launch_bounds__(kTileThreads)
   predict_tile_kernel(const T* __restrict__ X, int64_t n_rows, int F, int pitch, int n_batches,
                       const BatchInfo* __restrict__ batches, const PackedTree* __restrict__ desc,
                       const PackedNode<T>* __restrict__ nodes, const double* __restrict__ leaves, int K,
                       double* __restrict__ out)
 {
+  using S = TileShape<L>;
+  constexpr int kTileRows = S::kRows, kLaneTrees = S::kLaneTrees;
   extern __shared__ unsigned char smem_raw[];
   T* s_x = reinterpret_cast<T*>(smem_raw);
   const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
@@ -338,8 +352,8 @@ __global__ void __launch_bounds__(kTileThreads)
       }
     }
   }
-  const int r      = threadIdx.x >> 2;
-  const int q      = threadIdx.x & 3;
+  const int r      = threadIdx.x / L;
+  const int q      = threadIdx.x & (L - 1);
   const bool valid = r < rows_here;
   const T* my_x    = s_x + (valid ? r : 0) * pitch;
   constexpr int kAcc = kSingle ? 1 : kTileMaxK;
@@ -350,7 +364,7 @@ __global__ void __launch_bounds__(kTileThreads)
   // fetched one batch ahead: the batch descriptor, the nodes (as 16-byte words) and where this
   // lane's trees start inside the batch
   BatchInfo info_n = batches[0];
-  Prefetched pf = fetch_batch<T>(info_n, nodes, desc, q);
+  Prefetched<S> pf = fetch_batch<T, S>(info_n, nodes, desc, q);
   double val[kLaneTrees];  // single output: leaf values of this lane's trees of the previous batch
   int cnt_prev = 0;
 #pragma unroll
@@ -376,7 +390,7 @@ __global__ void __launch_bounds__(kTileThreads)
     __syncthreads();
     if (b + 1 < n_batches) {
       info_n = batches[b + 1];
-      pf = fetch_batch<T>(info_n, nodes, desc, q);
+      pf = fetch_batch<T, S>(info_n, nodes, desc, q);
     }
     for (int s = 0; s < info.steps; s++) {
 #pragma unroll
@@ -394,7 +408,7 @@ __global__ void __launch_bounds__(kTileThreads)
     if constexpr (kSingle) {
       // leaf values of the previous batch arrived while this one was walked: every lane of the
       // four forms the same sum, in tree order
-      add_in_order(acc[0], val, cnt_prev);
+      add_in_order<S>(acc[0], val, cnt_prev);
 #pragma unroll
       for (int j = 0; j < kLaneTrees; j++) val[j] = leaves[info.node_off + base[j] + pos[j]];
       cnt_prev = info.count;
@@ -402,10 +416,10 @@ __global__ void __launch_bounds__(kTileThreads)
       int at[kLaneTrees];
 #pragma unroll
       for (int j = 0; j < kLaneTrees; j++) at[j] = base[j] + pos[j];
-      add_leaves_in_order<kAcc>(acc, at, info.count, leaves + info.node_off * K, K);
+      add_leaves_in_order<S, kAcc>(acc, at, info.count, leaves + info.node_off * K, K);
     }
   }
-  if constexpr (kSingle) add_in_order(acc[0], val, cnt_prev);
+  if constexpr (kSingle) add_in_order<S>(acc[0], val, cnt_prev);
   if (valid && q == 0) {
     double* o = out + (row0 + r) * K;
 #pragma unroll
@@ -436,9 +450,21 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
 {
   *done = false;
   if (workspace == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
-  const int pitch      = F | 1;  // odd pitch: the rows of a wave start in different LDS banks
-  const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
-  if (x_bytes + 4096 > kTileLds) return LBT_OK;
+  const int pitch = F | 1;  // odd pitch: the rows of a wave start in different LDS banks
+  // lanes per row: as few as keep the row tile within about half of the LDS
+  int lanes      = 0;
+  size_t x_bytes = 0;
+  for (int l : {4, 8, 16}) {
+    x_bytes = (static_cast<size_t>(kTileThreads / l) * pitch * sizeof(T) + 15) & ~size_t(15);
+    if (x_bytes <= kTileLds * 55 / 100) {
+      lanes = l;
+      break;
+    }
+  }
+  if (lanes == 0) return LBT_OK;
+  const int tile_rows   = kTileThreads / lanes;
+  const int batch_trees = lanes == 4 ? TileShape<4>::kBatchTrees
+                                     : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees);
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
   const int64_t node_cap = std::min<int64_t>(static_cast<int64_t>((kTileLds - x_bytes) / sizeof(PackedNode<T>)),
                                              static_cast<int64_t>(kCopyWords) * kTileThreads * kNodesPerWord);
@@ -463,7 +489,7 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   const size_t node_bytes  = (padded_nodes(n_trees, total_nodes) * sizeof(PackedNode<T>) + 255) & ~size_t(255);
   double* leaves           = reinterpret_cast<double*>(raw + desc_bytes + batch_bytes + node_bytes);
 
-  // batches: consecutive trees, at most kBatchTrees, whose nodes fit the LDS share together
+  // batches: consecutive trees, at most batch_trees, whose nodes fit the LDS share together
   std::vector<BatchInfo> binfo;
   std::vector<int64_t> node_off(n_trees);
   std::vector<int32_t> rel_off(n_trees);
@@ -474,7 +500,7 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
     bi.node_off = off;
     bi.first    = t;
     int64_t in_batch = 0;
-    while (t < n_trees && bi.count < kBatchTrees && in_batch + tree_nodes[t] <= node_cap) {
+    while (t < n_trees && bi.count < batch_trees && in_batch + tree_nodes[t] <= node_cap) {
       node_off[t] = off + in_batch;
       rel_off[t]  = static_cast<int32_t>(in_batch);
       int steps   = 0;
@@ -512,16 +538,20 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
     for (int i = 0; i < n; i++) tb.b[i] = binfo[first + i];
     write_batches_kernel<<<1, kPackBatches, 0, stream>>>(tb, first, n, batches);
   }
-  static bool attr_single[kMaxDevices] = {}, attr_multi[kMaxDevices] = {};
-  LBT_TRY(allow_dynamic_lds(predict_tile_kernel<T, true>, kTileLds, attr_single));
-  LBT_TRY(allow_dynamic_lds(predict_tile_kernel<T, false>, kTileLds, attr_multi));
-  const unsigned tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
-  if (K == 1)
-    predict_tile_kernel<T, true><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
-                                                                            nodes, leaves, K, out);
+  const unsigned tiles = static_cast<unsigned>((N + tile_rows - 1) / tile_rows);
+  auto launch = [&](auto kernel, bool (&flags)[kMaxDevices]) -> int {
+    LBT_TRY(allow_dynamic_lds(kernel, kTileLds, flags));
+    kernel<<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc, nodes, leaves, K, out);
+    return LBT_OK;
+  };
+  static bool attr[6][kMaxDevices] = {};
+  const bool single = K == 1;
+  if (lanes == 4)
+    LBT_TRY(single ? launch(predict_tile_kernel<T, true, 4>, attr[0]) : launch(predict_tile_kernel<T, false, 4>, attr[1]));
+  else if (lanes == 8)
+    LBT_TRY(single ? launch(predict_tile_kernel<T, true, 8>, attr[2]) : launch(predict_tile_kernel<T, false, 8>, attr[3]));
   else
-    predict_tile_kernel<T, false><<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc,
-                                                                             nodes, leaves, K, out);
+    LBT_TRY(single ? launch(predict_tile_kernel<T, true, 16>, attr[4]) : launch(predict_tile_kernel<T, false, 16>, attr[5]));
   LBT_HIP(hipGetLastError());
   *done = true;
   return LBT_OK;

@@ -187,15 +187,17 @@ def test_predict_matches_oracle_multi_tree_multi_output():
     assert np.array_equal(gu.cpu(ops.predict(X, [], 3)), np.zeros((30000, 3)))
 
 
-def test_predict_tiled_and_per_node_paths_agree_with_oracle():
-    """Mixed tree sizes, a feature count that is not a multiple of four, a row count that is not a
-    multiple of the tile, thresholds that equal feature values or sit between two floats."""
+@pytest.mark.parametrize("f,k", [(13, 1), (100, 1), (200, 3), (330, 1)])
+def test_predict_tiled_and_per_node_paths_agree_with_oracle(f, k):
+    """Mixed tree sizes, feature counts that take 4, 8 or 16 lanes per row (one not a multiple of
+    four), a row count that is not a multiple of the tile, thresholds that equal feature values or
+    sit between two floats."""
     import gpu_util as gu
     import oracle_lib as orc
     from lbtree import ops
 
     rs = np.random.RandomState(5)
-    n, f = 70001, 13
+    n = 70001 if f < 100 else 9001
     X = rs.rand(n, f).astype(np.float32)
     trees_c, trees_g = [], []
     for t in range(47):
@@ -211,16 +213,16 @@ def test_predict_tiled_and_per_node_paths_agree_with_oracle():
         vals = X[rs.randint(0, n, m), np.maximum(feat, 0)].astype(np.float64)
         split[::3] = vals[::3]
         split[::5] = vals[::5] + 1e-12
-        leaf = rs.randn(m, 1) * 0.01
+        leaf = rs.randn(m, k) * 0.01
         trees_c.append((leaf, feat, split))
         trees_g.append((ops.as_device(leaf), ops.as_device(feat), ops.as_device(split)))
-    want = orc.predict(X, trees_c, 1)
-    tiled = gu.cpu(ops.predict(X, trees_g, 1))
-    plain = gu.cpu(ops.predict(X, trees_g, 1, tiled=False))
+    want = orc.predict(X, trees_c, k)
+    tiled = gu.cpu(ops.predict(X, trees_g, k))
+    plain = gu.cpu(ops.predict(X, trees_g, k, tiled=False))
     assert np.array_equal(tiled, want)
     assert np.array_equal(plain, want)
     X64 = X.astype(np.float64) + 1e-13
-    assert np.array_equal(gu.cpu(ops.predict(X64, trees_g, 1)), orc.predict(X64, trees_c, 1))
+    assert np.array_equal(gu.cpu(ops.predict(X64, trees_g, k)), orc.predict(X64, trees_c, k))
 
 
 def test_update_tree_matches_oracle_within_rounding():
