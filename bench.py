@@ -159,7 +159,7 @@ def bench_training(args):
         else:
             # same values as PredictTask on the training rows (checked bit for bit in the tests)
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True)
-            pred.add_(r.leaf_value[r.row_leaf.long()])
+            pred.add_(r.leaf_value.index_select(0, r.row_leaf))
         return r
 
     def loss():
