@@ -926,7 +926,7 @@ struct Layout {
   RecInfo* rec;
   void* binned;
   size_t binned_bytes;
-  uint16_t* tables;
+  uint32_t* tables;
   void* cell_lo;
   void* cell_invw;
   // quantiser
@@ -988,7 +988,7 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
   L.binned_bytes = max_depth >= 2 ? static_cast<size_t>(N) * bin_row_bytes_max(F, S) : 0;
   L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(L.binned_bytes + 16)) : nullptr;
-  L.tables       = ar.take<uint16_t>(static_cast<size_t>(F) * kMaxCells);
+  L.tables       = ar.take<uint32_t>(static_cast<size_t>(F) * kMaxCells / 16);
   L.cell_lo      = ar.take<double>(F);
   L.cell_invw    = ar.take<double>(F);
   int64_t n_chunks = (N * K + 4095) / 4096;

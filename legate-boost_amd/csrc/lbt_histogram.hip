@@ -153,13 +153,26 @@ __device__ inline int cell_of(double x, double nlo, double invw, double cmax)
   return static_cast<int>(t);
 }
 
-// One workgroup per feature. table[c] = number of the feature's proposals
-// whose cell is < c. A value in cell c is >= every proposal in earlier cells
-// and < every proposal in later cells, so its lower bound lies at or after
-// table[c] and is found by probing forward while proposal < x.
+// Lookup table of a feature: the value range is cut into C fine cells (many more than there
+// are proposals) and the table holds one 32-bit word per 16 cells: the number of proposals in
+// all earlier words (high half) and a bit per cell of the word that holds at least one
+// proposal (low half). For a value in cell c,
+//   start = count(word of c) + popcount(bits of the word below c)
+// never exceeds the number of proposals below the value (a proposal in an earlier cell is
+// smaller than every value of a later cell, and a cell with several proposals is counted
+// once), so the lower bound lies at or after start and is found by comparing the next few
+// proposals; with 8 cells per proposal three comparisons almost always suffice.
+// One workgroup per feature, one thread per table word.
+constexpr int kCellsPerWord = 16;
+
+__device__ inline int table_start(uint32_t word, int cell)
+{
+  return static_cast<int>(word >> 16) + __popc(word & ((1u << (cell & (kCellsPerWord - 1))) - 1u));
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
-  build_cells_kernel(const T* proposals, const int32_t* row_pointers, int C, uint16_t* tables, T* lo_out,
+  build_cells_kernel(const T* proposals, const int32_t* row_pointers, int C, uint32_t* tables, T* lo_out,
                      T* invw_out)
 {
   __shared__ T s_lo, s_invw;
@@ -190,21 +203,29 @@ __global__ void __launch_bounds__(256)
     invw_out[f] = invw;
   }
   __syncthreads();
-  const T lo = s_lo, invw = s_invw, cmax = static_cast<T>(C - 1);
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    // first b with cell(p[b]) >= c
+  const T nlo = s_lo, invw = s_invw, cmax = static_cast<T>(C - 1);
+  const int words = C / kCellsPerWord;
+  for (int w = threadIdx.x; w < words; w += blockDim.x) {
+    // first proposal whose cell is >= the first cell of the word (the cells of the ascending
+    // proposals ascend too)
+    const int c0 = w * kCellsPerWord;
     int a = 0, len = n;
     while (len > 0) {
       int half = len >> 1;
-      if (cell_of(p[a + half], lo, invw, cmax) < c) {
+      if (cell_of(p[a + half], nlo, invw, cmax) < c0) {
         a += half + 1;
         len -= half + 1;
       } else {
         len = half;
       }
     }
-    // the +inf proposal sits in the last cell, so a <= n - 1 for every c <= C-1
-    tables[static_cast<int64_t>(f) * C + c] = static_cast<uint16_t>(a < n ? a : n - 1);
+    uint32_t bits = 0;
+    for (int i = a; i < n; i++) {
+      const int c = cell_of(p[i], nlo, invw, cmax);
+      if (c >= c0 + kCellsPerWord) break;
+      bits |= 1u << (c - c0);
+    }
+    tables[static_cast<int64_t>(f) * words + w] = (static_cast<uint32_t>(a) << 16) | bits;
   }
 }
 
@@ -273,7 +294,7 @@ struct HistArgs {
   const T* proposals;
   const int32_t* row_pointers;
   const int32_t* groups;  // feature groups: [n_groups+1]
-  const uint16_t* tables;
+  const uint32_t* tables;
   const T* cell_lo;
   const T* cell_invw;
   int cells;
@@ -360,18 +381,17 @@ __global__ void __launch_bounds__(kHistThreads)
 
   unsigned long long* s_hist = reinterpret_cast<unsigned long long*>(smem_raw);
   T* s_prop                  = reinterpret_cast<T*>(smem_raw + static_cast<size_t>(nb) * 8);
-  uint16_t* s_cell           = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(nb) * (8 + sizeof(T)));
+  uint32_t* s_cell           = reinterpret_cast<uint32_t*>(smem_raw + static_cast<size_t>(nb) * (8 + sizeof(T)));
 
   for (int i = threadIdx.x; i < nb; i += kHistThreads) {
     s_prop[i] = a.proposals[bin0 + i];
     s_hist[i] = 0;
   }
   {
-    // tables of the group's features are contiguous: copy as 32-bit words
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(a.tables + static_cast<int64_t>(f0) * C);
-    uint32_t* dst       = reinterpret_cast<uint32_t*>(s_cell);
-    const int words     = gs * C / 2;
-    for (int i = threadIdx.x; i < words; i += kHistThreads) dst[i] = src[i];
+    // tables of the group's features are contiguous
+    const uint32_t* src = a.tables + static_cast<int64_t>(f0) * (C / kCellsPerWord);
+    const int words     = gs * (C / kCellsPerWord);
+    for (int i = threadIdx.x; i < words; i += kHistThreads) s_cell[i] = src[i];
   }
 
   const int lanes_per_row = (gs + VEC - 1) / VEC;
@@ -387,7 +407,7 @@ __global__ void __launch_bounds__(kHistThreads)
     int f     = min(f0 + fl + v, f1 - 1);
     c_lo[v]   = a.cell_lo[f];
     c_invw[v] = a.cell_invw[f];
-    c_cell[v] = (f - f0) * C;
+    c_cell[v] = (f - f0) * (C / kCellsPerWord);
     c_prop[v] = a.row_pointers[f] - bin0;
     c_end[v]  = a.row_pointers[f + 1] - bin0;
   }
@@ -498,7 +518,8 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
           const T x = xs[v];
-          int bn = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
+          const int cell = cell_of(x, c_lo[v], c_invw[v], cmax);
+          int bn         = c_prop[v] + table_start(s_cell[c_cell[v] + cell / kCellsPerWord], cell);
           bool lt    = s_prop[bn] < x;
           int probes = 0;
           while (__any(lt)) {
@@ -556,7 +577,7 @@ struct BinRowsArgs {
   const int32_t* row_pointers;
   const int32_t* bin_feature;  // [bins] feature of every proposal
   const int32_t* sgroups;      // search groups: [n_sgroups+1]
-  const uint16_t* tables;
+  const uint32_t* tables;
   const T* cell_lo;
   const T* cell_invw;
   int cells;
@@ -590,7 +611,7 @@ __global__ void __launch_bounds__(kHistThreads)
   // entries, so a window of probes that starts anywhere in a feature stays ascending
   T* s_prop        = reinterpret_cast<T*>(smem_raw);
   const int np     = nb + kProbePad * gs + kProbeSlack;
-  uint16_t* s_cell = reinterpret_cast<uint16_t*>(smem_raw + static_cast<size_t>(np) * sizeof(T));
+  uint32_t* s_cell = reinterpret_cast<uint32_t*>(smem_raw + static_cast<size_t>(np) * sizeof(T));
   for (int i = threadIdx.x; i < nb; i += kHistThreads)
     s_prop[i + kProbePad * (a.bin_feature[bin0 + i] - f0)] = a.proposals[bin0 + i];
   for (int i = threadIdx.x; i < kProbePad * gs + kProbeSlack; i += kHistThreads) {
@@ -598,10 +619,9 @@ __global__ void __launch_bounds__(kHistThreads)
     s_prop[a.row_pointers[f0 + f + 1] - bin0 + kProbePad * f + (i - kProbePad * f)] = std::numeric_limits<T>::infinity();
   }
   {
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(a.tables + static_cast<int64_t>(f0) * C);
-    uint32_t* dst       = reinterpret_cast<uint32_t*>(s_cell);
-    const int words     = gs * C / 2;
-    for (int i = threadIdx.x; i < words; i += kHistThreads) dst[i] = src[i];
+    const uint32_t* src = a.tables + static_cast<int64_t>(f0) * (C / kCellsPerWord);
+    const int words     = gs * (C / kCellsPerWord);
+    for (int i = threadIdx.x; i < words; i += kHistThreads) s_cell[i] = src[i];
   }
   // group widths are multiples of VEC, so every lane owns VEC real features
   const int lanes_per_row = gs / VEC;
@@ -616,7 +636,7 @@ __global__ void __launch_bounds__(kHistThreads)
     const int f = fb + v;
     c_lo[v]   = a.cell_lo[f];
     c_invw[v] = a.cell_invw[f];
-    c_cell[v] = (f - f0) * C;
+    c_cell[v] = (f - f0) * (C / kCellsPerWord);
     c_prop[v] = a.row_pointers[f] - bin0 + kProbePad * (f - f0);
     c_end[v]  = a.row_pointers[f + 1] - bin0 + kProbePad * (f - f0);
   }
@@ -691,27 +711,28 @@ __global__ void __launch_bounds__(kHistThreads)
           xs[3] = x_c[u].w;
         }
         BinT rel[VEC];
-        // the table gives the first proposal the value can reach; the proposals from there on
+        // the table gives a proposal at or before the value's bin; the proposals from there on
         // are ascending, so the bin is that start plus the number of proposals below the value.
-        // Four of them are compared at once, without a branch; the (rare) lanes that saw four
+        // Three of them are compared at once, without a branch; the (rare) lanes that saw three
         // smaller proposals look at four more, and then finish with a binary search.
         int bn[VEC], cnt[VEC];
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
-          const T x   = xs[v];
-          bn[v]       = c_prop[v] + s_cell[c_cell[v] + cell_of(x, c_lo[v], c_invw[v], cmax)];
-          const T* pp = s_prop + bn[v];
-          cnt[v]      = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0) + (pp[3] < x ? 1 : 0);
+          const T x      = xs[v];
+          const int cell = cell_of(x, c_lo[v], c_invw[v], cmax);
+          bn[v]          = c_prop[v] + table_start(s_cell[c_cell[v] + cell / kCellsPerWord], cell);
+          const T* pp    = s_prop + bn[v];
+          cnt[v]         = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0);
         }
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
-          if (__any(cnt[v] == 4)) {
+          if (__any(cnt[v] == 3)) {
             const T x   = xs[v];
-            const T* pp = s_prop + bn[v] + 4;
+            const T* pp = s_prop + bn[v] + 3;
             const int c2 = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0) + (pp[3] < x ? 1 : 0);
-            cnt[v] += cnt[v] == 4 ? c2 : 0;
-            if (__any(cnt[v] == 8)) {
-              const int left = cnt[v] == 8 ? c_end[v] - (bn[v] + 8) : 0;
+            cnt[v] += cnt[v] == 3 ? c2 : 0;
+            if (__any(cnt[v] == 7)) {
+              const int left = cnt[v] == 7 ? c_end[v] - (bn[v] + 7) : 0;
               cnt[v] += count_less(pp + 4, left, x, a.search_steps);
             }
           }
@@ -1273,7 +1294,8 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   // sub-histogram when the same kernel accumulates (cache off). Histogram side with the
   // cache: the packed sub-histogram only.
   auto search_bytes = [&](int f, int cells) {
-    return static_cast<size_t>(rp[f + 1] - rp[f]) * (cached ? elem : 8 + elem) + static_cast<size_t>(cells) * 2 +
+    return static_cast<size_t>(rp[f + 1] - rp[f]) * (cached ? elem : 8 + elem) +
+           static_cast<size_t>(cells) / kCellsPerWord * sizeof(uint32_t) +
            (cached ? kProbePad * elem : 0);
   };
   auto hist_bytes = [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; };
@@ -1299,7 +1321,7 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   // ... then the largest table, up to four cells per proposal, that still fits these groups
   int cells = 64;
   size_t search_lds = widest_group(sgroups, [&](int f) { return search_bytes(f, 64); });
-  for (int c = 128; c <= kMaxCells && c <= 4 * std::max(16, max_feature_bins); c <<= 1) {
+  for (int c = 128; c <= kMaxCells && c <= 8 * std::max(16, max_feature_bins); c <<= 1) {
     const size_t need = widest_group(sgroups, [&](int f) { return search_bytes(f, c); });
     if (need > search_budget) break;
     cells      = c;

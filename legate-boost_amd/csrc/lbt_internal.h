@@ -300,7 +300,7 @@ struct HistSetup {
   // device buffers (carved from the caller's workspace)
   int32_t* groups    = nullptr;  // [n_groups + 1]
   int32_t* sgroups   = nullptr;  // [n_sgroups + 1]; the same array as groups when the cache is off
-  uint16_t* tables   = nullptr;  // [n_features][cells]
+  uint32_t* tables   = nullptr;  // [n_features][cells / 16]: one word per 16 cells
   void* cell_lo      = nullptr;  // X dtype [n_features]
   void* cell_invw    = nullptr;  // X dtype [n_features]
   int32_t* tile_start = nullptr;
@@ -327,7 +327,7 @@ struct HistSetup {
   int brpp             = 0;        // rows per workgroup pass, histogram kernel on cached bins
 };
 
-constexpr int kMaxCells = 2048;
+constexpr int kMaxCells = 16384;  // table cells per feature at most (one 32-bit word per 16 cells)
 constexpr int kHistThreads       = 1024;
 // LDS a histogram-stage workgroup may fill; 4 KB of the 160 KB stay free for the tile window
 constexpr size_t kLdsBudget = 160 * 1024 - 512 - 4096;
