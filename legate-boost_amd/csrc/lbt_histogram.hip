@@ -164,6 +164,7 @@ __device__ inline int cell_of(double x, double nlo, double invw, double cmax)
 // proposals; with 8 cells per proposal three comparisons almost always suffice.
 // One workgroup per feature, one thread per table word.
 constexpr int kCellsPerWord = 16;
+constexpr int kCellShift    = 4;  // log2(kCellsPerWord); cells are never negative
 
 __device__ inline int table_start(uint32_t word, int cell)
 {
@@ -519,7 +520,7 @@ __global__ void __launch_bounds__(kHistThreads)
         for (int v = 0; v < VEC; v++) {
           const T x = xs[v];
           const int cell = cell_of(x, c_lo[v], c_invw[v], cmax);
-          int bn         = c_prop[v] + table_start(s_cell[c_cell[v] + cell / kCellsPerWord], cell);
+          int bn         = c_prop[v] + table_start(s_cell[c_cell[v] + (static_cast<unsigned>(cell) >> kCellShift)], cell);
           bool lt    = s_prop[bn] < x;
           int probes = 0;
           while (__any(lt)) {
@@ -720,7 +721,7 @@ __global__ void __launch_bounds__(kHistThreads)
         for (int v = 0; v < VEC; v++) {
           const T x      = xs[v];
           const int cell = cell_of(x, c_lo[v], c_invw[v], cmax);
-          bn[v]          = c_prop[v] + table_start(s_cell[c_cell[v] + cell / kCellsPerWord], cell);
+          bn[v]          = c_prop[v] + table_start(s_cell[c_cell[v] + (static_cast<unsigned>(cell) >> kCellShift)], cell);
           const T* pp    = s_prop + bn[v];
           cnt[v]         = (pp[0] < x ? 1 : 0) + (pp[1] < x ? 1 : 0) + (pp[2] < x ? 1 : 0);
         }
