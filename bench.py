@@ -142,24 +142,30 @@ def bench_training(args):
         pred = torch.full((n, 1), float(y.mean()), dtype=torch.float64, device=X.device)
         yc = y.reshape(-1, 1)
 
+    gh = (torch.empty_like(pred), torch.empty_like(pred))
+
     def one_round():
-        if n_classes:
-            p = torch.softmax(pred, dim=1)
-            g = p.clone()
-            g[ar, label] -= 1.0
-            g *= lr
-            h = torch.clamp(p * (1.0 - p), min=1e-8)
-        else:
-            g = (pred - yc) * lr
-            h = torch.ones_like(pred)
         seed = int(rs.randint(0, 2**31))
         if args.reference_flow:
+            # the caller's steps as separate array operations and a traversal of X per round
+            if n_classes:
+                p = torch.softmax(pred, dim=1)
+                g = p.clone()
+                g[ar, label] -= 1.0
+                g *= lr
+                h = torch.clamp(p * (1.0 - p), min=1e-8)
+            else:
+                g = (pred - yc) * lr
+                h = torch.ones_like(pred)
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
             pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
         else:
-            # same values as PredictTask on the training rows (checked bit for bit in the tests)
+            # gradient step in one pass; the prediction update takes the rows' leaves from the
+            # build: same values as PredictTask on the training rows (checked bit for bit in the tests)
+            g, h = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc, pred,
+                                         None, lr, out=gh)
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True)
-            pred.add_(r.leaf_value.index_select(0, r.row_leaf))
+            ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         return r
 
     def loss():

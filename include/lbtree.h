@@ -146,6 +146,59 @@ int lbt_update_tree(void* stream, const void* X, int32_t x_dtype, int64_t n_rows
                     double l1_regularization, double l2_regularization, double* leaf_out,
                     double* hessian_out, void* workspace, size_t workspace_bytes);
 
+/* ---- the steps of a boosting round either side of BuildTreeTask ------------ */
+
+/* Objectives of lbt_weighted_gradient. */
+#define LBT_OBJ_SQUARED_ERROR 0 /* legateboost/objectives.py:131-147 */
+#define LBT_OBJ_LOG_LOSS 1      /* legateboost/objectives.py:489-531 */
+
+/*
+ * LBBase._get_weighted_gradient (legateboost/legateboost.py:189-224) for the two objectives
+ * above, in one pass over the rows instead of one cupynumeric task per operator:
+ *   p = transform(pred); (g, h) = gradient(y, p)
+ *   g = (g * w) * learning_rate;  h = max(h * w, 1e-8)
+ * with every product and difference rounded on its own, in that order.
+ *   pred    device double [n_rows][n_outputs], the raw (untransformed) predictions
+ *   y       device double: [n_rows][n_outputs] for squared error and for log loss with one
+ *           output (labels 0/1); [n_rows] class labels for log loss with several outputs
+ *   sample_weight  device double [n_rows], or NULL for all ones
+ *   g, h    device double [n_rows][n_outputs]; overwritten (may not alias pred or y)
+ * Squared error is exact. Log loss calls exp, which differs from numpy's in the last bit,
+ * and sums the softmax denominator in column order. Subsampling
+ * (legateboost.py:213-220) is not part of this call.
+ */
+int lbt_weighted_gradient(void* stream, int32_t objective, const double* pred, const double* y,
+                          const double* sample_weight, double learning_rate, int64_t n_rows,
+                          int32_t n_outputs, double* g, double* h);
+
+/*
+ * pred[r][k] += leaf_value[row_leaf[r]][k]: the update `train_pred += model.predict(X)` of
+ * legateboost/legateboost.py:268 for the tree just built, from lbt_build_taps.row_leaf
+ * instead of a fresh traversal of X. Same doubles, same single addition per element as
+ * PredictTask followed by the caller's +=.
+ *   leaf_value  device double [n_nodes][n_outputs]
+ *   row_leaf    device int32 [n_rows], every entry in [0, n_nodes)
+ *   pred        device double [n_rows][n_outputs], updated in place
+ */
+int lbt_add_leaf_values(void* stream, const double* leaf_value, int32_t n_nodes,
+                        const int32_t* row_leaf, int64_t n_rows, int32_t n_outputs, double* pred);
+
+/*
+ * GatherTask::gpu_variant (src/utils/gather.cu:26-91), one GPU's share: row i of `out` is
+ * global row sample_rows[i] of X if this shard holds it, else zeros (the reference then
+ * sums the shards' outputs; with one shard that sum is the identity).
+ *   X             device [n_rows][n_features], dtype x_dtype, global rows
+ *                 [row_offset, row_offset + n_rows)
+ *   sample_rows   n_samples global row numbers: a HOST array if samples_on_host is non-zero
+ *                 (the task's scalar form, gather.cu:47-60), else a device array
+ *   staging       device int64 [n_samples] when samples_on_host is non-zero (the copy of
+ *                 sample_rows that the kernel reads); ignored otherwise
+ *   out           device [n_samples][n_features], dtype x_dtype; overwritten
+ */
+int lbt_gather_rows(void* stream, const void* X, int32_t x_dtype, int64_t row_offset, int64_t n_rows,
+                    int32_t n_features, const int64_t* sample_rows, int64_t n_samples,
+                    int32_t samples_on_host, int64_t* staging, void* out);
+
 /* ---- profiling (no counterpart in the reference) -------------------------- */
 
 #define LBT_PROF_PROPOSALS 0

@@ -14,6 +14,8 @@ LBT_OK = 0
 LBT_F32 = 0
 LBT_F64 = 1
 LBT_MAX_SPLIT_SAMPLES = 2048
+LBT_OBJ_SQUARED_ERROR = 0
+LBT_OBJ_LOG_LOSS = 1
 PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "positions", "other", "predict", "binning"]
 
 
@@ -97,6 +99,15 @@ def _load():
     lib.lbt_update_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p,
                                     C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_double, C.c_void_p,
                                     C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_weighted_gradient.restype = C.c_int
+    lib.lbt_weighted_gradient.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
+                                          C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.lbt_add_leaf_values.restype = C.c_int
+    lib.lbt_add_leaf_values.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int32,
+                                        C.c_void_p]
+    lib.lbt_gather_rows.restype = C.c_int
+    lib.lbt_gather_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_void_p,
+                                    C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
     lib.lbt_profile_enable.restype = None
     lib.lbt_profile_enable.argtypes = [C.c_int]
     lib.lbt_profile_reset.restype = None
@@ -110,7 +121,8 @@ lib = _load()
 EXPORTS = [
     "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_predict",
     "lbt_predict_workspace_bytes",
-    "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_profile_enable", "lbt_profile_reset",
+    "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
+    "lbt_gather_rows", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",
 ]
 

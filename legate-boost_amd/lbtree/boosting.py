@@ -22,6 +22,8 @@ def _check_random_state(seed):
 
 
 class SquaredErrorObjective:
+    fused = "squared_error"  # ops.weighted_gradient computes transform + gradient + weighting in one pass
+
     def gradient(self, y, pred):
         return pred - y, torch.ones_like(pred)
 
@@ -35,6 +37,8 @@ class SquaredErrorObjective:
 
 
 class LogLossObjective:
+    fused = "log_loss"
+
     def gradient(self, y, pred):
         if pred.shape[1] == 1:
             return pred - y, pred * (1.0 - pred)
@@ -94,6 +98,9 @@ class LBBase:
         return X, y
 
     def _get_weighted_gradient(self, y, pred, sample_weight, learning_rate):
+        fused = getattr(self._objective_instance, "fused", None)
+        if fused is not None and pred.is_cuda:
+            return ops.weighted_gradient(fused, y, pred, sample_weight, learning_rate)
         g, h = self._objective_instance.gradient(y, self._objective_instance.transform(pred))
         g = g * sample_weight[:, None] * learning_rate
         h = torch.clamp(h * sample_weight[:, None], min=1e-8)
@@ -121,10 +128,12 @@ class LBBase:
         train_pred = self._predict(X)
         for i in range(self.n_estimators):
             g, h = self._get_weighted_gradient(y, train_pred, w, self.learning_rate)
-            self.models_.append(
-                deepcopy(self.base_models[i % len(self.base_models)]).set_random_state(self.random_state_).fit(X, g, h)
-            )
-            train_pred += self.models_[-1].predict(X)
+            model = deepcopy(self.base_models[i % len(self.base_models)]).set_random_state(self.random_state_)
+            if hasattr(model, "fit_update_predictions"):
+                model.fit_update_predictions(X, g, h, train_pred)
+            else:
+                train_pred += model.fit(X, g, h).predict(X)
+            self.models_.append(model)
             if self.verbose:
                 print("i: {} train loss: {:.6f}".format(i, self._loss(y, train_pred, w)))
         self._train_pred = train_pred

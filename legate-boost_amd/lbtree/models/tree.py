@@ -61,6 +61,15 @@ class Tree(BaseModel):
         return id * 2 + 2
 
     def fit(self, X, g, h) -> "Tree":
+        return self._fit(X, g, h, None)
+
+    def fit_update_predictions(self, X, g, h, pred) -> "Tree":
+        """`fit(X, g, h)` followed by `pred += self.predict(X)` (legateboost/legateboost.py:262-268)
+        without the second pass over X: the build records the leaf of every training row, and
+        pred (CUDA float64 [n_rows, n_outputs], updated in place) receives that leaf's value."""
+        return self._fit(X, g, h, pred)
+
+    def _fit(self, X, g, h, pred) -> "Tree":
         X = ops.as_device(X)
         n_features = X.shape[1]
         # the seed is drawn before the feature sample, as in tree.py:125 / :139-157
@@ -81,8 +90,10 @@ class Tree(BaseModel):
         r = ops.build_tree(
             X, g, h, max_depth=self.max_depth, split_samples=self.split_samples, seed=seed,
             l1_regularization=self.l1_regularization, l2_regularization=self.l2_regularization,
-            min_split_gain=self.min_split_gain, feature_set=feature_set,
+            min_split_gain=self.min_split_gain, feature_set=feature_set, row_leaf=pred is not None,
         )
+        if pred is not None:
+            ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         self.leaf_value = r.leaf_value
         self.feature = r.feature
         self.split_value = r.split_value

@@ -195,3 +195,74 @@ def update_tree(X, g, h, feature, split_value, l1_regularization, l2_regularizat
                                   l2_regularization, leaf.data_ptr(), hess.data_ptr(), ws.data_ptr(), ws.numel())
     _lib.check(rc)
     return leaf, hess
+
+
+_OBJECTIVES = {"squared_error": _lib.LBT_OBJ_SQUARED_ERROR, "log_loss": _lib.LBT_OBJ_LOG_LOSS}
+
+
+def weighted_gradient(objective, y, pred, sample_weight=None, learning_rate=1.0, out=None):
+    """LBBase._get_weighted_gradient (legateboost/legateboost.py:189-224) for "squared_error" or
+    "log_loss" in one pass. pred: raw predictions [n, K]; y: [n, K], or [n] / [n, 1] class labels
+    for log loss with K > 1. Returns (g, h); `out=(g, h)` reuses two buffers of pred's shape."""
+    pred = as_device(pred, torch.float64)
+    y = as_device(y, torch.float64)
+    if pred.dim() != 2:
+        raise _lib.LbtError("pred must be [n_rows, n_outputs]")
+    n, k = pred.shape
+    labels = objective == "log_loss" and k > 1
+    if y.numel() != (n if labels else n * k):
+        raise _lib.LbtError("y has %d elements, expected %d" % (y.numel(), n if labels else n * k))
+    w = None
+    if sample_weight is not None:
+        w = as_device(sample_weight, torch.float64)
+        if w.numel() != n:
+            raise _lib.LbtError("sample_weight must have one entry per row")
+    if objective not in _OBJECTIVES:
+        raise _lib.LbtError("unknown objective %r" % (objective,))
+    g, h = out if out is not None else (torch.empty_like(pred), torch.empty_like(pred))
+    rc = _lib.lib.lbt_weighted_gradient(_stream(), _OBJECTIVES[objective], pred.data_ptr(), y.data_ptr(),
+                                        w.data_ptr() if w is not None else None, float(learning_rate), n, k,
+                                        g.data_ptr(), h.data_ptr())
+    _lib.check(rc)
+    return g, h
+
+
+def add_leaf_values(pred, leaf_value, row_leaf):
+    """pred += leaf_value[row_leaf], in place: the caller's `train_pred += tree.predict(X)`
+    (legateboost/legateboost.py:268) from the rows' leaves recorded by build_tree(row_leaf=True)."""
+    if not (pred.is_cuda and pred.dtype == torch.float64 and pred.is_contiguous() and pred.dim() == 2):
+        raise _lib.LbtError("pred must be a contiguous CUDA float64 [n_rows, n_outputs] tensor")
+    leaf_value = as_device(leaf_value, torch.float64)
+    row_leaf = as_device(row_leaf, torch.int32)
+    n, k = pred.shape
+    if leaf_value.dim() != 2 or leaf_value.shape[1] != k or row_leaf.numel() != n:
+        raise _lib.LbtError("leaf_value must be [n_nodes, n_outputs] and row_leaf [n_rows]")
+    rc = _lib.lib.lbt_add_leaf_values(_stream(), leaf_value.data_ptr(), leaf_value.shape[0], row_leaf.data_ptr(), n, k,
+                                      pred.data_ptr())
+    _lib.check(rc)
+    return pred
+
+
+def gather_rows(X, samples, row_offset=0):
+    """GATHER (legateboost/utils.py:412-460, src/utils/gather.cu:26-91): rows `samples` (global
+    numbers) of X; rows this shard does not hold come back as zeros. samples: a tuple / numpy
+    array (sent as the task's host scalar) or a CUDA int64 tensor."""
+    X = _check_x(X)
+    n, f = X.shape
+    on_host = not (isinstance(samples, torch.Tensor) and samples.is_cuda)
+    if on_host:
+        rows = np.ascontiguousarray(np.asarray(samples, dtype=np.int64).reshape(-1))
+        m = rows.shape[0]
+        staging = torch.empty(max(m, 1), dtype=torch.int64, device=X.device)
+        rows_p, staging_p = rows.ctypes.data, staging.data_ptr()
+    else:
+        rows = samples.to(torch.int64).contiguous().reshape(-1)
+        m = rows.shape[0]
+        rows_p, staging_p = rows.data_ptr(), None
+    out = torch.empty((m, f), dtype=X.dtype, device=X.device)
+    rc = _lib.lib.lbt_gather_rows(_stream(), X.data_ptr(), _DT[X.dtype], row_offset, n, f, rows_p, m, int(on_host),
+                                  staging_p, out.data_ptr())
+    _lib.check(rc)
+    if on_host:
+        torch.cuda.current_stream().synchronize()  # the host array is read by the copy on the stream
+    return out

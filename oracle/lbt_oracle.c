@@ -747,3 +747,68 @@ void orc_update_tree(const void* X, int is64, int64_t n_rows, int32_t F, const d
     leaf_out[i] = H[i] > 0.0 ? orc_calculate_leaf_value(G[i], H[i], l1, l2) : 0.0;
   free(G);
 }
+
+/* ------------------------------------------------------------------------- */
+/* The boosting round's steps around the tree build                            */
+/* ------------------------------------------------------------------------- */
+
+/* legateboost.py:205-211: weights, learning rate and the floor of the hessian */
+static void weigh(double g0, double h0, double w, double lr, double* g, double* h)
+{
+  double hw = h0 * w;
+  *g        = (g0 * w) * lr;
+  *h        = hw > 1e-8 ? hw : 1e-8;
+}
+
+void orc_weighted_gradient(int32_t objective, const double* pred, const double* y,
+                           const double* weight, double lr, int64_t n_rows, int32_t K, double* g,
+                           double* h)
+{
+  for (int64_t r = 0; r < n_rows; r++) {
+    double w = weight ? weight[r] : 1.0;
+    if (objective == 0) {
+      /* objectives.py:131-132: pred - y, ones */
+      for (int k = 0; k < K; k++)
+        weigh(pred[r * K + k] - y[r * K + k], 1.0, w, lr, &g[r * K + k], &h[r * K + k]);
+    } else if (K == 1) {
+      /* objectives.py:492-493 after the sigmoid of :507-508 */
+      double p = 1.0 / (1.0 + exp(-pred[r]));
+      weigh(p - y[r], p * (1.0 - p), w, lr, &g[r], &h[r]);
+    } else {
+      /* softmax objectives.py:510-514, then :496-501 */
+      double top = pred[r * K];
+      for (int k = 1; k < K; k++)
+        if (pred[r * K + k] > top) top = pred[r * K + k];
+      double div = 0.0;
+      for (int k = 0; k < K; k++) div += exp(pred[r * K + k] - top);
+      int label = (int)y[r];
+      for (int k = 0; k < K; k++) {
+        double p  = exp(pred[r * K + k] - top) / div;
+        double g0 = k == label ? p + -1.0 : p;
+        weigh(g0, p * (1.0 - p), w, lr, &g[r * K + k], &h[r * K + k]);
+      }
+    }
+  }
+}
+
+void orc_add_leaf_values(const double* leaf, const int32_t* row_leaf, int64_t n_rows, int32_t K,
+                         double* pred)
+{
+  for (int64_t r = 0; r < n_rows; r++)
+    for (int k = 0; k < K; k++) pred[r * K + k] += leaf[(int64_t)row_leaf[r] * K + k];
+}
+
+void orc_gather_rows(const void* X, int is64, int64_t row_offset, int64_t n_rows, int32_t F,
+                     const int64_t* rows, int64_t n_samples, void* out)
+{
+  for (int64_t i = 0; i < n_samples; i++) {
+    int64_t row = rows[i] - row_offset;
+    int has     = row >= 0 && row < n_rows;
+    for (int j = 0; j < F; j++) {
+      if (is64)
+        ((double*)out)[i * F + j] = has ? ((const double*)X)[row * F + j] : 0.0;
+      else
+        ((float*)out)[i * F + j] = has ? ((const float*)X)[row * F + j] : 0.0f;
+    }
+  }
+}

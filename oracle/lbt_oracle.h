@@ -28,6 +28,9 @@
  *                                        "parity unpinned"
  *   positions .......................... pinned (brute-force stable sort)
  *   predict / update ................... pinned (brute force, closed forms)
+ *   weighted gradient .................. pinned (closed forms; the known answers of
+ *                                        the reference's test_objective.py::test_log_loss)
+ *   add leaf values / gather rows ...... pinned (numpy indexing)
  */
 #ifndef LBT_ORACLE_H
 #define LBT_ORACLE_H
@@ -138,6 +141,21 @@ void orc_update_tree(const void* X, int x_is_f64, int64_t n_rows, int32_t n_feat
                      const double* g, const double* h, int32_t n_outputs,
                      const int32_t* feature, const double* split, int32_t n_nodes, double l1,
                      double l2, double* leaf_out, double* hessian_out);
+
+/* legateboost/legateboost.py:189-224 on top of objectives.py:131-147 (objective 0, squared
+ * error) or :489-531 (objective 1, log loss). pred holds raw predictions [n_rows][K]; y is
+ * [n_rows][K], or [n_rows] class labels for log loss with K > 1; weight is [n_rows] or NULL. */
+void orc_weighted_gradient(int32_t objective, const double* pred, const double* y,
+                           const double* weight, double learning_rate, int64_t n_rows,
+                           int32_t n_outputs, double* g, double* h);
+
+/* legateboost.py:268 for one tree, from the rows' leaves: pred[r][k] += leaf[row_leaf[r]][k]. */
+void orc_add_leaf_values(const double* leaf, const int32_t* row_leaf, int64_t n_rows,
+                         int32_t n_outputs, double* pred);
+
+/* src/utils/gather.cu:67-73: out[i][j] = X[rows[i]][j] if this shard holds the row, else 0. */
+void orc_gather_rows(const void* X, int x_is_f64, int64_t row_offset, int64_t n_rows,
+                     int32_t n_features, const int64_t* rows, int64_t n_samples, void* out);
 
 #ifdef __cplusplus
 }

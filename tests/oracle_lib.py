@@ -95,6 +95,14 @@ def _load():
     lib.orc_update_tree.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p,
                                     C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_double,
                                     C.c_void_p, C.c_void_p]
+    lib.orc_weighted_gradient.restype = None
+    lib.orc_weighted_gradient.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_int64,
+                                          C.c_int32, C.c_void_p, C.c_void_p]
+    lib.orc_add_leaf_values.restype = None
+    lib.orc_add_leaf_values.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]
+    lib.orc_gather_rows.restype = None
+    lib.orc_gather_rows.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int64,
+                                    C.c_void_p]
     return lib
 
 
@@ -265,3 +273,34 @@ def update_tree(X, g, h, feature, split, l1, l2):
     hess = np.empty((m, k), np.float64)
     lib.orc_update_tree(_p(X), is64, n, f, _p(g), _p(h), k, _p(feature), _p(split), m, l1, l2, _p(leaf), _p(hess))
     return leaf, hess
+
+
+OBJECTIVES = {"squared_error": 0, "log_loss": 1}
+
+
+def weighted_gradient(objective, y, pred, weight=None, learning_rate=1.0):
+    pred = np.ascontiguousarray(pred, np.float64)
+    y = np.ascontiguousarray(y, np.float64)
+    n, k = pred.shape
+    w = None if weight is None else np.ascontiguousarray(weight, np.float64)
+    g = np.empty_like(pred)
+    h = np.empty_like(pred)
+    lib.orc_weighted_gradient(OBJECTIVES[objective], _p(pred), _p(y), None if w is None else _p(w),
+                              learning_rate, n, k, _p(g), _p(h))
+    return g, h
+
+
+def add_leaf_values(pred, leaf, row_leaf):
+    pred = np.array(pred, np.float64, order="C")
+    leaf = np.ascontiguousarray(leaf, np.float64)
+    row_leaf = np.ascontiguousarray(row_leaf, np.int32)
+    lib.orc_add_leaf_values(_p(leaf), _p(row_leaf), pred.shape[0], pred.shape[1], _p(pred))
+    return pred
+
+
+def gather_rows(X, rows, row_offset=0):
+    X, is64 = _check_x(X)
+    rows = np.ascontiguousarray(rows, np.int64)
+    out = np.empty((rows.shape[0], X.shape[1]), X.dtype)
+    lib.orc_gather_rows(_p(X), is64, row_offset, X.shape[0], X.shape[1], _p(rows), rows.shape[0], _p(out))
+    return out

@@ -72,6 +72,17 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert rc == -1
     rc = _lib.lib.lbt_predict(None, one, 9, 10, 2, 0, None, None, None, None, 1, one, None, 0)
     assert rc == -1
+    two = C.c_void_p(32)
+    rc = _lib.lib.lbt_weighted_gradient(None, 7, one, one, None, 1.0, 10, 1, two, two)
+    assert rc == -1 and b"objective" in _lib.lib.lbt_last_error()
+    rc = _lib.lib.lbt_weighted_gradient(None, _lib.LBT_OBJ_SQUARED_ERROR, one, two, None, 1.0, 10, 1, one, two)
+    assert rc == -1 and b"alias" in _lib.lib.lbt_last_error()
+    assert _lib.lib.lbt_weighted_gradient(None, _lib.LBT_OBJ_LOG_LOSS, None, None, None, 1.0, 0, 3, None, None) == 0
+    assert _lib.lib.lbt_add_leaf_values(None, one, 0, one, 10, 1, one) == -1
+    assert _lib.lib.lbt_add_leaf_values(None, None, 3, None, 0, 1, None) == 0
+    assert _lib.lib.lbt_gather_rows(None, one, 3, 0, 10, 2, one, 4, 0, None, one) == -1
+    rc = _lib.lib.lbt_gather_rows(None, one, _lib.LBT_F32, 0, 10, 2, one, 4, 1, None, one)
+    assert rc == -1 and b"staging" in _lib.lib.lbt_last_error()
     with pytest.raises(_lib.LbtError):
         _lib.check(rc)
 

@@ -239,6 +239,75 @@ def test_update_tree_matches_oracle_within_rounding():
     assert np.allclose(gu.cpu(hess_g), hess_c, rtol=1e-9)
 
 
+@pytest.mark.parametrize("k", [1, 3])
+def test_squared_error_gradient_is_bit_exact(k):
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(40 + k)
+    n = 100003
+    pred, y, w = rs.normal(size=(n, k)), rs.normal(size=(n, k)), rs.gamma(2.0, size=n)
+    w[:3] = [0.0, 1e-12, 1e6]
+    for weight in (None, w):
+        g_c, h_c = orc.weighted_gradient("squared_error", y, pred, weight, 0.3)
+        g_g, h_g = ops.weighted_gradient("squared_error", y, pred, weight, 0.3)
+        assert np.array_equal(gu.cpu(g_g), g_c) and np.array_equal(gu.cpu(h_g), h_c)
+
+
+@pytest.mark.parametrize("k", [1, 2, 8, 13])
+def test_log_loss_gradient_matches_oracle(k):
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(50 + k)
+    n = 50021
+    pred = 5 * rs.normal(size=(n, k))
+    pred[0] = 700.0 * (1 - 2 * (np.arange(k) % 2))  # saturated row
+    y = rs.randint(0, max(k, 2), n).astype(np.float64)
+    w = rs.gamma(2.0, size=n)
+    g_c, h_c = orc.weighted_gradient("log_loss", y.reshape(-1, 1) if k == 1 else y, pred, w, 0.1)
+    g_g, h_g = ops.weighted_gradient("log_loss", y.reshape(-1, 1) if k == 1 else y, pred, w, 0.1)
+    # the device's exp and libm's differ in the last bit: 1e-12 of the largest gradient of the row
+    scale = np.abs(g_c).max(axis=1, keepdims=True) + 1e-300
+    assert (np.abs(gu.cpu(g_g) - g_c) <= 1e-12 * scale).all()
+    assert np.allclose(gu.cpu(h_g), h_c, rtol=1e-12, atol=0)
+    assert np.isfinite(gu.cpu(g_g)).all() and (gu.cpu(h_g) >= 1e-8).all()
+
+
+@pytest.mark.parametrize("k", [1, 4])
+def test_row_leaf_prediction_update_equals_predict(k):
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    X, g, h = _problem(60 + k, 30000, 9, k)
+    r = ops.build_tree(X, g, h, max_depth=6, split_samples=64, seed=3, row_leaf=True)
+    base = np.random.RandomState(1).normal(size=(30000, k))
+    pred = torch.from_numpy(base.copy()).cuda()
+    ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
+    tree = (r.leaf_value, r.feature, r.split_value)
+    assert torch.equal(pred, torch.from_numpy(base).cuda() + ops.predict(X, [tree], k))
+    assert np.array_equal(gu.cpu(pred), orc.add_leaf_values(base, gu.cpu(r.leaf_value), gu.cpu(r.row_leaf)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gather_rows_matches_oracle(dtype):
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(8)
+    X = rs.normal(size=(5000, 17)).astype(dtype)
+    rows = rs.randint(900, 6200, 300).astype(np.int64)  # some outside the shard [1000, 6000)
+    want = orc.gather_rows(X, rows, row_offset=1000)
+    assert (want == 0).all(axis=1).any() and (want != 0).any()
+    assert np.array_equal(gu.cpu(ops.gather_rows(X, tuple(rows), row_offset=1000)), want)
+    assert np.array_equal(gu.cpu(ops.gather_rows(X, torch.from_numpy(rows).cuda(), row_offset=1000)), want)
+    assert ops.gather_rows(X, (), row_offset=0).shape == (0, 17)
+
+
 def test_two_runs_are_bit_identical():
     import gpu_util as gu
 

@@ -529,3 +529,83 @@ def test_update_after_fit_reproduces_fit():
     assert np.allclose(leaf[used], r.leaf_value[used], rtol=1e-4, atol=1e-6)
     assert np.allclose(hess[used], r.hessian[used], rtol=1e-5)
     assert (leaf[~used] == 0).all()
+
+
+# ---- the boosting round's steps around the tree build ----------------------------------------
+
+
+def test_reference_log_loss_known_answers():
+    # legateboost/test/test_objective.py::test_log_loss gives gradient() probabilities; the raw
+    # predictions that transform() maps to them are their logits / logarithms
+    g, h = orc.weighted_gradient("log_loss", np.array([[1.0], [0.0]]), np.zeros((2, 1)))
+    assert np.allclose(g, [[-0.5], [0.5]]) and np.allclose(h, [[0.25], [0.25]])
+    prob = np.array([[0.3, 0.3, 0.4], [0.3, 0.4, 0.3], [0.4, 0.3, 0.3]])
+    g, h = orc.weighted_gradient("log_loss", np.array([2.0, 1.0, 0.0]), np.log(prob) + 7.0)
+    assert np.allclose(g, [[0.3, 0.3, -0.6], [0.3, -0.6, 0.3], [-0.6, 0.3, 0.3]])
+    assert np.allclose(h, [[0.21, 0.21, 0.24], [0.21, 0.24, 0.21], [0.24, 0.21, 0.21]])
+
+
+def test_weighted_gradient_against_the_reference_operator_sequence():
+    # legateboost.py:205-211 spelt out with numpy, operator by operator
+    rs = np.random.RandomState(11)
+    n = 257
+    w = rs.gamma(2.0, size=n)
+    w[:5] = [0.0, 1e-12, 1.0, 3.0, 1e6]
+    lr = 0.3
+    for k in (1, 3):
+        pred, y = rs.normal(size=(n, k)), rs.normal(size=(n, k))
+        g, h = orc.weighted_gradient("squared_error", y, pred, w, lr)
+        assert np.array_equal(g, (pred - y) * w[:, None] * lr)
+        assert np.array_equal(h, np.maximum(np.ones((n, k)) * w[:, None], 1e-8))
+        g, h = orc.weighted_gradient("squared_error", y, pred, None, lr)
+        assert np.array_equal(g, (pred - y) * 1.0 * lr) and np.array_equal(h, np.ones((n, k)))
+    pred, y = 4 * rs.normal(size=(n, 1)), rs.randint(0, 2, (n, 1)).astype(np.float64)
+    p = 1.0 / (1.0 + np.exp(-pred))
+    g, h = orc.weighted_gradient("log_loss", y, pred, w, lr)
+    assert np.allclose(g, (p - y) * w[:, None] * lr, rtol=1e-13, atol=0)
+    assert np.allclose(h, np.maximum(p * (1 - p) * w[:, None], 1e-8), rtol=1e-13, atol=0)
+    assert h.min() == 1e-8  # the zero-weight rows sit on the floor
+    k = 5
+    pred, lab = 6 * rs.normal(size=(n, k)), rs.randint(0, k, n)
+    pred[7] = [800.0, -800.0, 0.0, 799.0, 1.0]  # no overflow thanks to the row maximum
+    e = np.exp(pred - pred.max(axis=1)[:, None])
+    p = e / e.sum(axis=1)[:, None]
+    gg = p.copy()
+    gg[np.arange(n), lab] -= 1.0
+    g, h = orc.weighted_gradient("log_loss", lab.astype(np.float64), pred, w, lr)
+    assert np.allclose(g, gg * w[:, None] * lr, rtol=1e-12, atol=1e-300)
+    assert np.allclose(h, np.maximum(p * (1 - p) * w[:, None], 1e-8), rtol=1e-12, atol=0)
+    assert np.isfinite(g).all() and np.isfinite(h).all()
+    # the class gradients of a row sum to zero, its hessians are those of a probability vector
+    g1, h1 = orc.weighted_gradient("log_loss", lab.astype(np.float64), pred)
+    assert np.abs(g1.sum(axis=1)).max() < 1e-15 and (h1 <= 0.25 + 1e-16).all()
+
+
+def test_add_leaf_values_and_gather_rows_are_plain_indexing():
+    rs = np.random.RandomState(5)
+    leaf = rs.normal(size=(31, 3))
+    row_leaf = rs.randint(0, 31, 500).astype(np.int32)
+    pred = rs.normal(size=(500, 3))
+    assert np.array_equal(orc.add_leaf_values(pred, leaf, row_leaf), pred + leaf[row_leaf])
+    for dt in (np.float32, np.float64):
+        X = rs.normal(size=(40, 7)).astype(dt)
+        rows = np.array([100, 139, 99, 140, 120, 120, -1], np.int64)
+        want = np.zeros((7, 7), dt)
+        want[[0, 1, 4, 5]] = X[[0, 39, 20, 20]]
+        assert np.array_equal(orc.gather_rows(X, rows, row_offset=100), want)
+
+
+def test_row_leaf_update_equals_predict():
+    # what the fused update relies on: leaf[row -> leaf] is PredictTask on the training rows
+    rs = np.random.RandomState(2)
+    X = rs.normal(size=(300, 6)).astype(np.float32)
+    g, h = rs.normal(size=(300, 2)), np.ones((300, 2))
+    t = orc.build_tree(X, g, h, max_depth=4, split_samples=16, seed=9)
+    pr = orc.predict(X, [(t.leaf_value, t.feature, t.split_value)], 2)
+    walk = np.zeros(300, np.int32)
+    for r in range(300):
+        nd = 0
+        while t.feature[nd] != -1:
+            nd = 2 * nd + 1 if X[r, t.feature[nd]] <= t.split_value[nd] else 2 * nd + 2
+        walk[r] = nd
+    assert np.array_equal(orc.add_leaf_values(np.zeros((300, 2)), t.leaf_value, walk), pr)
