@@ -131,6 +131,45 @@ int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, in
                 const double* const* split, const int32_t* tree_nodes, int32_t n_outputs,
                 double* out, void* workspace, size_t workspace_bytes);
 
+/*
+ * The packed ensemble as an object of its own: pack once, predict many batches. This is the
+ * form lbt_predict builds in its workspace on every call: per tree one array of 8-byte
+ * (float X) or 16-byte (double X) nodes holding threshold, feature and right child, leaves
+ * marked by a NaN threshold, trees grouped into batches that share the LDS, and the leaf
+ * values beside them. It replaces the 3 * n_trees task inputs of legateboost/models/tree.py:264-273
+ * for callers that predict repeatedly with one model (no counterpart in the reference).
+ * The descriptor is host memory owned by the caller; `data` is the caller's device buffer.
+ */
+typedef struct lbt_packed_ensemble {
+  void* data;   /* device buffer passed to lbt_pack_ensemble */
+  size_t bytes; /* its size */
+  int32_t x_dtype;
+  int32_t n_features;
+  int32_t n_outputs;
+  int32_t n_trees;
+  int32_t n_batches; /* groups of trees that are staged in the LDS together */
+  int32_t lanes;     /* lanes that share a row in the traversal kernel (4, 8 or 16; set by n_features) */
+  int64_t total_nodes;
+} lbt_packed_ensemble;
+
+/*
+ * Packs n_trees trees (arguments as for lbt_predict) for X of the given dtype and width into
+ * `buffer` (device, at least lbt_predict_workspace_bytes(n_trees, total_nodes, n_outputs, x_dtype))
+ * and fills *ensemble. The trees' own arrays are not referenced after the stream has passed
+ * this call. Returns LBT_ERR_UNSUPPORTED when the shapes do not fit the packed form (more
+ * than 8 outputs, a tree of more than 65535 nodes or too large for the LDS, rows too wide):
+ * lbt_predict without a workspace serves those.
+ */
+int lbt_pack_ensemble(void* stream, int32_t x_dtype, int32_t n_features, int32_t n_trees,
+                      const double* const* leaf, const int32_t* const* feature, const double* const* split,
+                      const int32_t* tree_nodes, int32_t n_outputs, void* buffer, size_t buffer_bytes,
+                      lbt_packed_ensemble* ensemble);
+
+/* PredictTask over a packed ensemble: out [n_rows][n_outputs] is overwritten with the same
+ * sums, added in tree order, as lbt_predict gives for the trees that were packed. */
+int lbt_predict_packed(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                       const lbt_packed_ensemble* ensemble, double* out);
+
 /* Device scratch needed by lbt_update_tree. */
 size_t lbt_update_tree_workspace_bytes(int64_t n_rows, int32_t n_outputs, int32_t n_nodes);
 

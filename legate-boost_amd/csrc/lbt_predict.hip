@@ -441,28 +441,51 @@ size_t packed_bytes(int n_trees, int64_t total_nodes, int K, size_t node_size)
          padded_nodes(n_trees, total_nodes) * static_cast<size_t>(K) * sizeof(double) + 512;
 }
 
-// Returns LBT_OK and sets *done when the tiled path ran; leaves *done false when the shapes
-// do not fit it (then the caller takes the per-node path).
+// Where the parts of a packed ensemble lie in its buffer.
 template <typename T>
-int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees, const double* const* leaf,
-                  const int32_t* const* feature, const double* const* split, const int32_t* tree_nodes, int K,
-                  double* out, void* workspace, size_t workspace_bytes, bool* done)
-{
-  *done = false;
-  if (workspace == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
-  const int pitch = F | 1;  // odd pitch: the rows of a wave start in different LDS banks
-  // lanes per row: as few as keep the row tile within about half of the LDS
-  int lanes      = 0;
-  size_t x_bytes = 0;
-  for (int l : {4, 8, 16}) {
-    x_bytes = (static_cast<size_t>(kTileThreads / l) * pitch * sizeof(T) + 15) & ~size_t(15);
-    if (x_bytes <= kTileLds * 55 / 100) {
-      lanes = l;
-      break;
-    }
+struct PackedLayout {
+  PackedTree* desc;
+  BatchInfo* batches;
+  PackedNode<T>* nodes;
+  double* leaves;
+  PackedLayout(void* buffer, int n_trees, int64_t total_nodes)
+  {
+    const size_t desc_bytes  = (static_cast<size_t>(n_trees) * sizeof(PackedTree) + 255) & ~size_t(255);
+    const size_t batch_bytes = (static_cast<size_t>(n_trees) * sizeof(BatchInfo) + 255) & ~size_t(255);
+    const size_t node_bytes  = (padded_nodes(n_trees, total_nodes) * sizeof(PackedNode<T>) + 255) & ~size_t(255);
+    uintptr_t raw            = (reinterpret_cast<uintptr_t>(buffer) + 255) & ~uintptr_t(255);
+    desc                     = reinterpret_cast<PackedTree*>(raw);
+    batches                  = reinterpret_cast<BatchInfo*>(raw + desc_bytes);
+    nodes                    = reinterpret_cast<PackedNode<T>*>(raw + desc_bytes + batch_bytes);
+    leaves                   = reinterpret_cast<double*>(raw + desc_bytes + batch_bytes + node_bytes);
   }
+};
+
+// Lanes per row of the tile kernel for rows of F values: as few as keep the row tile within
+// about half of the LDS; 0 when no shape fits.
+template <typename T>
+int tile_lanes(int F, size_t* x_bytes)
+{
+  const int pitch = F | 1;  // odd pitch: the rows of a wave start in different LDS banks
+  for (int l : {4, 8, 16}) {
+    *x_bytes = (static_cast<size_t>(kTileThreads / l) * pitch * sizeof(T) + 15) & ~size_t(15);
+    if (*x_bytes <= kTileLds * 55 / 100) return l;
+  }
+  return 0;
+}
+
+// Packs the trees for the tile kernel into `buffer`. Returns LBT_OK and fills *ens when the
+// shapes fit the tile kernel; leaves ens->data null when they do not.
+template <typename T>
+int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf, const int32_t* const* feature,
+               const double* const* split, const int32_t* tree_nodes, int K, void* buffer, size_t buffer_bytes,
+               lbt_packed_ensemble* ens)
+{
+  *ens = lbt_packed_ensemble{};
+  if (buffer == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
+  size_t x_bytes  = 0;
+  const int lanes = tile_lanes<T>(F, &x_bytes);
   if (lanes == 0) return LBT_OK;
-  const int tile_rows   = kTileThreads / lanes;
   const int batch_trees = lanes == 4 ? TileShape<4>::kBatchTrees
                                      : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees);
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
@@ -476,18 +499,11 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   }
   if (max_nodes > node_cap || max_nodes > kMaxPackedNodes) return LBT_OK;
   const size_t need = packed_bytes(n_trees, total_nodes, K, sizeof(PackedNode<T>));
-  if (workspace_bytes < need) {
-    set_error("predict workspace too small: %zu bytes given, %zu needed", workspace_bytes, need);
+  if (buffer_bytes < need) {
+    set_error("packed ensemble buffer too small: %zu bytes given, %zu needed", buffer_bytes, need);
     return LBT_ERR_WORKSPACE;
   }
-  const size_t desc_bytes  = (static_cast<size_t>(n_trees) * sizeof(PackedTree) + 255) & ~size_t(255);
-  const size_t batch_bytes = (static_cast<size_t>(n_trees) * sizeof(BatchInfo) + 255) & ~size_t(255);
-  uintptr_t raw            = (reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255);
-  PackedTree* desc         = reinterpret_cast<PackedTree*>(raw);
-  BatchInfo* batches       = reinterpret_cast<BatchInfo*>(raw + desc_bytes);
-  PackedNode<T>* nodes     = reinterpret_cast<PackedNode<T>*>(raw + desc_bytes + batch_bytes);
-  const size_t node_bytes  = (padded_nodes(n_trees, total_nodes) * sizeof(PackedNode<T>) + 255) & ~size_t(255);
-  double* leaves           = reinterpret_cast<double*>(raw + desc_bytes + batch_bytes + node_bytes);
+  PackedLayout<T> lay(buffer, n_trees, total_nodes);
 
   // batches: consecutive trees, at most batch_trees, whose nodes fit the LDS share together
   std::vector<BatchInfo> binfo;
@@ -514,7 +530,6 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
     off += in_batch;
     binfo.push_back(bi);
   }
-  ProfScope ps(LBT_PROF_PREDICT, stream, static_cast<double>(N) * (static_cast<double>(F) * sizeof(T) + K * 8.0));
   for (int first = 0; first < n_trees; first += kPackTrees) {
     PackBatch b{};
     const int n = std::min(kPackTrees, n_trees - first);
@@ -529,19 +544,42 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
       widest         = std::max(widest, tree_nodes[first + i]);
     }
     dim3 grid(static_cast<unsigned>((widest + 255) / 256), n);
-    pack_trees_kernel<T><<<grid, 256, 0, stream>>>(b, first, F, K, desc, nodes, leaves);
+    pack_trees_kernel<T><<<grid, 256, 0, stream>>>(b, first, F, K, lay.desc, lay.nodes, lay.leaves);
   }
   const int n_batches = static_cast<int>(binfo.size());
   for (int first = 0; first < n_batches; first += kPackBatches) {
     BatchTable tb{};
     const int n = std::min(kPackBatches, n_batches - first);
     for (int i = 0; i < n; i++) tb.b[i] = binfo[first + i];
-    write_batches_kernel<<<1, kPackBatches, 0, stream>>>(tb, first, n, batches);
+    write_batches_kernel<<<1, kPackBatches, 0, stream>>>(tb, first, n, lay.batches);
   }
+  LBT_HIP(hipGetLastError());
+  ens->data        = buffer;
+  ens->bytes       = buffer_bytes;
+  ens->x_dtype     = sizeof(T) == 4 ? LBT_F32 : LBT_F64;
+  ens->n_features  = F;
+  ens->n_outputs   = K;
+  ens->n_trees     = n_trees;
+  ens->n_batches   = n_batches;
+  ens->lanes       = lanes;
+  ens->total_nodes = total_nodes;
+  return LBT_OK;
+}
+
+// The tile kernel over a packed ensemble.
+template <typename T>
+int run_tiled(hipStream_t stream, const T* X, int64_t N, const lbt_packed_ensemble& ens, double* out)
+{
+  const int F = ens.n_features, K = ens.n_outputs, lanes = ens.lanes, n_batches = ens.n_batches;
+  PackedLayout<T> lay(ens.data, ens.n_trees, ens.total_nodes);
+  const int pitch     = F | 1;
+  const int tile_rows = kTileThreads / lanes;
+  ProfScope ps(LBT_PROF_PREDICT, stream, static_cast<double>(N) * (static_cast<double>(F) * sizeof(T) + K * 8.0));
   const unsigned tiles = static_cast<unsigned>((N + tile_rows - 1) / tile_rows);
   auto launch = [&](auto kernel, bool (&flags)[kMaxDevices]) -> int {
     LBT_TRY(allow_dynamic_lds(kernel, kTileLds, flags));
-    kernel<<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, batches, desc, nodes, leaves, K, out);
+    kernel<<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes,
+                                                      lay.leaves, K, out);
     return LBT_OK;
   };
   static bool attr[6][kMaxDevices] = {};
@@ -553,6 +591,21 @@ int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees,
   else
     LBT_TRY(single ? launch(predict_tile_kernel<T, true, 16>, attr[4]) : launch(predict_tile_kernel<T, false, 16>, attr[5]));
   LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
+// Returns LBT_OK and sets *done when the tiled path ran; leaves *done false when the shapes
+// do not fit it (then the caller takes the per-node path).
+template <typename T>
+int predict_tiled(hipStream_t stream, const T* X, int64_t N, int F, int n_trees, const double* const* leaf,
+                  const int32_t* const* feature, const double* const* split, const int32_t* tree_nodes, int K,
+                  double* out, void* workspace, size_t workspace_bytes, bool* done)
+{
+  *done = false;
+  lbt_packed_ensemble ens;
+  LBT_TRY(pack_tiled<T>(stream, F, n_trees, leaf, feature, split, tree_nodes, K, workspace, workspace_bytes, &ens));
+  if (ens.data == nullptr) return LBT_OK;
+  LBT_TRY(run_tiled<T>(stream, X, N, ens, out));
   *done = true;
   return LBT_OK;
 }
@@ -696,6 +749,59 @@ int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, in
   if (done) return LBT_OK;
   return lbt::predict_impl<double>(s, static_cast<const double*>(X), n_rows, n_features, n_trees, leaf,
                                    feature, split, tree_nodes, n_outputs, out);
+}
+
+int lbt_pack_ensemble(void* stream, int32_t x_dtype, int32_t n_features, int32_t n_trees,
+                      const double* const* leaf, const int32_t* const* feature, const double* const* split,
+                      const int32_t* tree_nodes, int32_t n_outputs, void* buffer, size_t buffer_bytes,
+                      lbt_packed_ensemble* ensemble)
+{
+  LBT_REQUIRE(ensemble != nullptr, "null ensemble descriptor");
+  *ensemble = lbt_packed_ensemble{};
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(n_features >= 1 && n_outputs >= 1 && n_trees >= 1, "bad shape");
+  LBT_REQUIRE(leaf && feature && split && tree_nodes, "null tree arrays");
+  for (int i = 0; i < n_trees; i++)
+    LBT_REQUIRE(leaf[i] && feature[i] && split[i] && tree_nodes[i] >= 1, "tree %d is incomplete", i);
+  if (buffer == nullptr) {
+    lbt::set_error("null buffer for the packed ensemble");
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (x_dtype == LBT_F32)
+    LBT_TRY(lbt::pack_tiled<float>(s, n_features, n_trees, leaf, feature, split, tree_nodes, n_outputs, buffer,
+                                   buffer_bytes, ensemble));
+  else
+    LBT_TRY(lbt::pack_tiled<double>(s, n_features, n_trees, leaf, feature, split, tree_nodes, n_outputs, buffer,
+                                    buffer_bytes, ensemble));
+  if (ensemble->data == nullptr) {
+    lbt::set_error("ensemble does not fit the packed form (more than %d outputs, more than 65535 features or "
+                   "nodes per tree, or rows too wide for the LDS): use lbt_predict", lbt::kTileMaxK);
+    return LBT_ERR_UNSUPPORTED;
+  }
+  return LBT_OK;
+}
+
+int lbt_predict_packed(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                       const lbt_packed_ensemble* ensemble, double* out)
+{
+  LBT_REQUIRE(ensemble != nullptr && ensemble->data != nullptr, "ensemble was not packed");
+  LBT_REQUIRE(x_dtype == ensemble->x_dtype && n_features == ensemble->n_features,
+              "X (dtype %d, %d features) does not match the packed ensemble (dtype %d, %d features)", x_dtype,
+              n_features, ensemble->x_dtype, ensemble->n_features);
+  LBT_REQUIRE((ensemble->lanes == 4 || ensemble->lanes == 8 || ensemble->lanes == 16) && ensemble->n_trees >= 1 &&
+                ensemble->n_batches >= 1 && ensemble->n_batches <= ensemble->n_trees &&
+                ensemble->n_outputs >= 1 && ensemble->n_outputs <= lbt::kTileMaxK &&
+                ensemble->total_nodes >= ensemble->n_trees,
+              "corrupt ensemble descriptor");
+  LBT_REQUIRE(ensemble->bytes >= lbt_predict_workspace_bytes(ensemble->n_trees, ensemble->total_nodes,
+                                                             ensemble->n_outputs, ensemble->x_dtype),
+              "corrupt ensemble descriptor (buffer size)");
+  if (n_rows < 1) return LBT_OK;
+  LBT_REQUIRE(X && out, "null X or output");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (x_dtype == LBT_F32) return lbt::run_tiled<float>(s, static_cast<const float*>(X), n_rows, *ensemble, out);
+  return lbt::run_tiled<double>(s, static_cast<const double*>(X), n_rows, *ensemble, out);
 }
 
 size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype)

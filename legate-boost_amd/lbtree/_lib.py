@@ -68,6 +68,20 @@ class Profile(C.Structure):
     ]
 
 
+class PackedEnsemble(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p),
+        ("bytes", C.c_size_t),
+        ("x_dtype", C.c_int32),
+        ("n_features", C.c_int32),
+        ("n_outputs", C.c_int32),
+        ("n_trees", C.c_int32),
+        ("n_batches", C.c_int32),
+        ("lanes", C.c_int32),
+        ("total_nodes", C.c_int64),
+    ]
+
+
 class LbtError(RuntimeError):
     """Raised for a non-zero status; the reference throws std::runtime_error at the same places."""
 
@@ -99,6 +113,12 @@ def _load():
     lib.lbt_update_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p,
                                     C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_double, C.c_void_p,
                                     C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_pack_ensemble.restype = C.c_int
+    lib.lbt_pack_ensemble.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
+                                      C.c_void_p, C.c_int32, C.c_void_p, C.c_size_t, C.POINTER(PackedEnsemble)]
+    lib.lbt_predict_packed.restype = C.c_int
+    lib.lbt_predict_packed.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
+                                       C.POINTER(PackedEnsemble), C.c_void_p]
     lib.lbt_weighted_gradient.restype = C.c_int
     lib.lbt_weighted_gradient.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
                                           C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
@@ -120,7 +140,7 @@ lib = _load()
 
 EXPORTS = [
     "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_predict",
-    "lbt_predict_workspace_bytes",
+    "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",

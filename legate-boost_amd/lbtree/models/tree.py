@@ -152,3 +152,61 @@ class Tree(BaseModel):
         new = copy.deepcopy(self)
         new.leaf_value = new.leaf_value * scalar
         return new
+
+    def onnx_attributes(self, output_idx: int = 0) -> dict:
+        """Attributes of the ai.onnx.ml TreeEnsemble (opset 5) operator that carries output
+        `output_idx` of this tree, as numpy arrays: the mapping of legateboost/models/tree.py:319-392.
+        Node i of the tree is interior node i and leaf i of the operator at once, so features,
+        thresholds and leaf values pass through unchanged; `nodes_modes` 0 is the "<=" comparison,
+        a true comparison goes to the left child 2i+1."""
+        feature = self.feature.cpu().numpy()
+        n = feature.shape[0]
+        ids = np.arange(n)
+        left, right = 2 * ids + 1, 2 * ids + 2
+        # children of the last level point past the array: clamp before asking whether they are leaves
+        is_leaf = feature == -1
+        return {
+            "n_targets": int(self.leaf_value.shape[1]),
+            "aggregate_function": 1,
+            "post_transform": 0,
+            "tree_roots": [0],
+            "nodes_modes": np.zeros(n, np.uint8),
+            "nodes_featureids": feature,
+            "nodes_splits": self.split_value.cpu().numpy(),
+            "nodes_truenodeids": left,
+            "nodes_trueleafs": is_leaf[np.minimum(n - 1, left)].astype(int),
+            "nodes_falsenodeids": right,
+            "nodes_falseleafs": is_leaf[np.minimum(n - 1, right)].astype(int),
+            "leaf_targetids": np.full(n, output_idx, np.int64),
+            "leaf_weights": self.leaf_value[:, output_idx].cpu().numpy(),
+        }
+
+    def to_onnx(self) -> Any:
+        """ONNX model of this tree (legateboost/models/tree.py:319-438): one TreeEnsemble operator
+        per output, their results added up. Needs the `onnx` package."""
+        import onnx
+        from onnx import TensorProto, helper, numpy_helper
+
+        n_outputs = int(self.leaf_value.shape[1])
+        nodes = []
+        for k in range(n_outputs):
+            a = self.onnx_attributes(k)
+            a["nodes_modes"] = helper.make_tensor("nodes_modes", TensorProto.UINT8, a["nodes_modes"].shape,
+                                                  a["nodes_modes"])
+            a["nodes_splits"] = numpy_helper.from_array(a["nodes_splits"])
+            a["leaf_weights"] = numpy_helper.from_array(a["leaf_weights"])
+            nodes.append(helper.make_node("TreeEnsemble", ["X"], ["pred%d" % k], domain="ai.onnx.ml",
+                                          membership_values=None, nodes_missing_value_tracks_true=None,
+                                          nodes_hitrates=None, **a))
+            if k == 0:
+                nodes.append(helper.make_node("Identity", ["pred0"], ["accumulated_pred0"]))
+            else:
+                nodes.append(helper.make_node("Add", ["accumulated_pred%d" % (k - 1), "pred%d" % k],
+                                              ["accumulated_pred%d" % k]))
+        out = helper.make_tensor_value_info("accumulated_pred%d" % (n_outputs - 1), TensorProto.DOUBLE, [None, None])
+        X = helper.make_tensor_value_info("X", TensorProto.DOUBLE, [None, None])
+        graph = helper.make_graph(nodes, "legateboost.models.Tree", [X], [out])
+        model = helper.make_model(graph, opset_imports=[helper.make_opsetid("ai.onnx.ml", 5),
+                                                        helper.make_opsetid("", 14)])
+        onnx.checker.check_model(model)
+        return model

@@ -144,6 +144,53 @@ def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0
     return r
 
 
+def _tree_arrays(trees, n_outputs):
+    nt = len(trees)
+    leaf_p = (C.c_void_p * max(nt, 1))()
+    feat_p = (C.c_void_p * max(nt, 1))()
+    split_p = (C.c_void_p * max(nt, 1))()
+    nodes = (C.c_int32 * max(nt, 1))()
+    keep = []
+    for i, (lv, ft, sp) in enumerate(trees):
+        lv = as_device(lv, torch.float64)
+        ft = as_device(ft, torch.int32)
+        sp = as_device(sp, torch.float64)
+        if lv.dim() != 2 or lv.shape[1] != n_outputs or ft.shape[0] != lv.shape[0] or sp.shape[0] != lv.shape[0]:
+            raise _lib.LbtError("tree %d has inconsistent shapes" % i)
+        keep.append((lv, ft, sp))
+        leaf_p[i], feat_p[i], split_p[i], nodes[i] = lv.data_ptr(), ft.data_ptr(), sp.data_ptr(), ft.shape[0]
+    return leaf_p, feat_p, split_p, nodes, keep
+
+
+class PackedEnsemble:
+    """An ensemble packed once for repeated prediction (lbt_pack_ensemble): owns the device
+    buffer and the descriptor; tied to the dtype and width of the X it will be applied to."""
+
+    def __init__(self, trees, n_outputs, n_features, dtype=torch.float32, device=None):
+        if dtype not in _DT:
+            raise _lib.LbtError("X must be float32 or float64, got %s" % dtype)
+        leaf_p, feat_p, split_p, nodes, keep = _tree_arrays(trees, n_outputs)
+        nt = len(trees)
+        total = sum(int(nodes[i]) for i in range(nt))
+        device = device if device is not None else (keep[0][0].device if keep else "cuda")
+        nbytes = int(_lib.lib.lbt_predict_workspace_bytes(nt, total, n_outputs, _DT[dtype]))
+        self.buffer = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        self.desc = _lib.PackedEnsemble()
+        self.dtype, self.n_features, self.n_outputs = dtype, n_features, n_outputs
+        rc = _lib.lib.lbt_pack_ensemble(_stream(), _DT[dtype], n_features, nt, leaf_p, feat_p, split_p, nodes,
+                                        n_outputs, self.buffer.data_ptr(), nbytes, C.byref(self.desc))
+        _lib.check(rc)
+
+    def predict(self, X):
+        X = _check_x(X)
+        n, f = X.shape
+        out = torch.empty((n, self.n_outputs), dtype=torch.float64, device=X.device)
+        rc = _lib.lib.lbt_predict_packed(_stream(), X.data_ptr(), _DT[X.dtype], n, f, C.byref(self.desc),
+                                         out.data_ptr())
+        _lib.check(rc)
+        return out
+
+
 def predict(X, trees, n_outputs, tiled=True):
     """PREDICT (legateboost/models/tree.py:245-280). trees: sequence of
     (leaf_value [nodes,K] f64, feature [nodes] i32, split_value [nodes] f64) CUDA tensors."""

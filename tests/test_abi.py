@@ -73,6 +73,10 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     rc = _lib.lib.lbt_predict(None, one, 9, 10, 2, 0, None, None, None, None, 1, one, None, 0)
     assert rc == -1
     two = C.c_void_p(32)
+    ens = _lib.PackedEnsemble()
+    assert _lib.lib.lbt_predict_packed(None, one, _lib.LBT_F32, 10, 2, C.byref(ens), one) == -1
+    assert b"not packed" in _lib.lib.lbt_last_error()
+    assert _lib.lib.lbt_pack_ensemble(None, _lib.LBT_F32, 2, 0, None, None, None, None, 1, one, 64, C.byref(ens)) == -1
     rc = _lib.lib.lbt_weighted_gradient(None, 7, one, one, None, 1.0, 10, 1, two, two)
     assert rc == -1 and b"objective" in _lib.lib.lbt_last_error()
     rc = _lib.lib.lbt_weighted_gradient(None, _lib.LBT_OBJ_SQUARED_ERROR, one, two, None, 1.0, 10, 1, one, two)

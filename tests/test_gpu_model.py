@@ -200,3 +200,38 @@ def test_classifier(num_class):
     proba = _np(m.predict_proba(X))
     assert proba.shape == (4000, num_class) and np.allclose(proba.sum(axis=1), 1.0)
     assert (_np(m.predict(X)) == y).mean() > 0.7
+
+
+def _tree_ensemble_eval(a, X):
+    """ai.onnx.ml TreeEnsemble (opset 5) for one tree with BRANCH_LEQ nodes and SUM aggregation."""
+    out = np.zeros((X.shape[0], a["n_targets"]))
+    for r in range(X.shape[0]):
+        i, leaf = a["tree_roots"][0], False
+        while not leaf:
+            assert a["nodes_modes"][i] == 0
+            if X[r, a["nodes_featureids"][i]] <= a["nodes_splits"][i]:
+                i, leaf = a["nodes_truenodeids"][i], bool(a["nodes_trueleafs"][i])
+            else:
+                i, leaf = a["nodes_falsenodeids"][i], bool(a["nodes_falseleafs"][i])
+        out[r, a["leaf_targetids"][i]] += a["leaf_weights"][i]
+    return out
+
+
+def test_onnx_attributes_describe_the_same_function():
+    import lbtree as lb
+
+    rs = np.random.RandomState(4)
+    X = rs.randn(400, 5)
+    g, h = rs.randn(400, 2), np.ones((400, 2))
+    tree = lb.models.Tree(max_depth=4, split_samples=32).set_random_state(np.random.RandomState(1)).fit(X, g, h)
+    assert _np(tree.feature)[0] != -1
+    want = _np(tree.predict(X))
+    got = sum(_tree_ensemble_eval(tree.onnx_attributes(k), X) for k in range(2))
+    assert np.array_equal(got, want)
+    try:
+        import onnx  # noqa: F401
+    except ImportError:
+        with pytest.raises(ImportError):
+            tree.to_onnx()
+    else:
+        assert tree.to_onnx().graph.name == "legateboost.models.Tree"

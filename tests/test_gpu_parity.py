@@ -225,6 +225,39 @@ def test_predict_tiled_and_per_node_paths_agree_with_oracle(f, k):
     assert np.array_equal(gu.cpu(ops.predict(X64, trees_g, k)), orc.predict(X64, trees_c, k))
 
 
+@pytest.mark.parametrize("f,k,dtype", [(13, 1, np.float32), (100, 3, np.float32), (330, 1, np.float32),
+                                       (40, 2, np.float64)])
+def test_packed_ensemble_predicts_like_the_oracle(f, k, dtype):
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import _lib, ops
+
+    rs = np.random.RandomState(f + k)
+    X = rs.normal(size=(4099, f)).astype(dtype)
+    trees = []
+    for t in range(37):
+        depth = 1 + t % 6
+        m = 2 ** (depth + 1) - 1
+        feature = np.full(m, -1, np.int32)
+        inner = 2 ** depth - 1
+        feature[:inner] = rs.randint(0, f, inner)
+        feature[rs.randint(1, max(inner, 2), 2)] = -1  # early leaves; their subtrees are unreachable
+        split = rs.normal(size=m)
+        split[:3] = X[:3, feature[0]]  # thresholds that equal feature values: <= goes left
+        trees.append((rs.normal(size=(m, k)), feature, split))
+    dev = [tuple(ops.as_device(a) for a in t) for t in trees]
+    ens = ops.PackedEnsemble(dev, k, f, torch.float32 if dtype == np.float32 else torch.float64)
+    want = orc.predict(X, trees, k)
+    for rows in (X, X[:1], X[:777]):  # the same packed ensemble serves batch after batch
+        got = gu.cpu(ens.predict(rows))
+        assert np.array_equal(got, want[: rows.shape[0]])
+    assert ens.predict(X[:0]).shape == (0, k)
+    with pytest.raises(_lib.LbtError, match="does not match"):
+        ens.predict(X[:, : f - 1])
+    with pytest.raises(_lib.LbtError, match="does not match"):
+        ens.predict(X.astype(np.float64 if dtype == np.float32 else np.float32))
+
+
 def test_update_tree_matches_oracle_within_rounding():
     import gpu_util as gu
     import oracle_lib as orc
