@@ -22,6 +22,7 @@
 #include "models/tree/build_tree.h"
 #include "models/tree/predict.h"
 #include "models/tree/update_tree.h"
+#include "utils/gather.h"
 
 namespace legateboost {
 namespace {
@@ -181,6 +182,36 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   check(lbt_update_tree(context.get_task_stream(), X, dtype, rows, static_cast<int>(xs.hi[1] - xs.lo[1] + 1), g, h,
                         outputs, feature, split, nodes, l1, l2, leaf, hessian, workspace.ptr(0), ws_bytes));
   workspace.destroy();
+}
+
+/*static*/ void GatherTask::gpu_variant(legate::TaskContext context)
+{
+  // src/utils/gather.cu:26-91: X is 2-dimensional here; the output holds one row per sample and is
+  // broadcast, the sample rows arrive as scalar 0 (host) or as input 1 (device)
+  const auto X_store = context.input(0).data();
+  legate::Rect<2> xs, os;
+  const int dtype    = x_dtype(X_store);
+  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 2>(X_store, &xs))
+                                        : static_cast<const void*>(dense_in<double, 2>(X_store, &xs));
+  const int64_t rows = std::max<int64_t>(xs.hi[0] - xs.lo[0] + 1, 0);
+  auto out_store     = context.output(0).data();
+  os                 = out_store.shape<2>();
+  size_t strides[2];
+  void* out = dtype == LBT_F32 ? static_cast<void*>(out_store.write_accessor<float, 2>().ptr(os, strides))
+                               : static_cast<void*>(out_store.write_accessor<double, 2>().ptr(os, strides));
+  const int features = static_cast<int>(os.hi[1] - os.lo[1] + 1);
+  if (!context.scalars().empty()) {
+    auto samples = context.scalar(0).values<int64_t>();
+    auto staging = legate::create_buffer<int64_t>(samples.size(), legate::Memory::GPU_FB_MEM);
+    check(lbt_gather_rows(context.get_task_stream(), X, dtype, xs.lo[0], rows, features, samples.data(),
+                          static_cast<int64_t>(samples.size()), 1, staging.ptr(0), out));
+  } else {
+    legate::Rect<1> ss;
+    const int64_t* samples = dense_in<int64_t, 1>(context.input(1).data(), &ss);
+    check(lbt_gather_rows(context.get_task_stream(), X, dtype, xs.lo[0], rows, features, samples,
+                          ss.hi[0] - ss.lo[0] + 1, 0, nullptr, out));
+  }
+  // more than one GPU: sum-all-reduce `out` over the shards here (gather.cu:76-80)
 }
 
 }  // namespace legateboost
