@@ -728,6 +728,112 @@ __global__ void __launch_bounds__(kThreads)
   row_leaf[p.y] = node;
 }
 
+// The same result, written window by window of the row space. The rows of a node ascend
+// along its segment (the partition is stable and starts from the identity), so the rows of
+// one window [w * kLeafWindow, (w + 1) * kLeafWindow) form one contiguous run in every
+// segment. A workgroup that takes all those runs writes a contiguous piece of row_leaf
+// whole, where the order of the segments scatters four bytes into a different cache line per row.
+constexpr int kLeafWindow   = 8192;     // rows per workgroup
+constexpr int kLeafThreads  = 1024;
+constexpr int kLeafParents  = 4096;     // segments a workgroup can index in its LDS
+constexpr int64_t kLeafBoundsEntries = int64_t(1) << 20;
+
+// bounds[j * (n_windows + 1) + w] = first index of segment j whose row is >= w * kLeafWindow
+__global__ void __launch_bounds__(kThreads)
+  leaf_window_bounds_kernel(const int2* pos, const int32_t* seg, int n_parents, int n_windows, int32_t* bounds)
+{
+  const int64_t t = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (t >= static_cast<int64_t>(n_parents) * (n_windows + 1)) return;
+  const int j = static_cast<int>(t / (n_windows + 1));
+  const int w = static_cast<int>(t - static_cast<int64_t>(j) * (n_windows + 1));
+  int lo = seg[j], hi = seg[j + 1];
+  if (w == n_windows) {
+    lo = hi;
+  } else if (w > 0) {
+    const int64_t first = static_cast<int64_t>(w) * kLeafWindow;
+    while (lo < hi) {
+      const int mid = lo + ((hi - lo) >> 1);
+      if (pos[mid].y < first)
+        lo = mid + 1;
+      else
+        hi = mid;
+    }
+  }
+  bounds[t] = lo;
+}
+
+template <typename BinT>
+__global__ void __launch_bounds__(kLeafThreads)
+  final_leaf_window_kernel(const int2* pos, const int32_t* bounds, int n_parents, int n_windows, int level_first,
+                           const BinT* bins_t, int64_t bins_stride, const int32_t* feature,
+                           const int32_t* split_bin, int32_t* row_leaf)
+{
+  __shared__ int s_lo[kLeafParents];
+  __shared__ int s_pre[kLeafParents + 1];  // exclusive prefix of the run lengths
+  __shared__ int s_wave[kLeafThreads / 64];
+  const int w = blockIdx.x;
+  // run of every segment in this window, four segments per thread
+  constexpr int kPer = kLeafParents / kLeafThreads;
+  int len[kPer];
+  int mine = 0;
+#pragma unroll
+  for (int u = 0; u < kPer; u++) {
+    const int j = threadIdx.x * kPer + u;
+    len[u]      = 0;
+    if (j < n_parents) {
+      const int32_t* b = bounds + static_cast<int64_t>(j) * (n_windows + 1) + w;
+      const int lo     = b[0];
+      s_lo[j]          = lo;
+      len[u]           = b[1] - lo;
+    }
+    mine += len[u];
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = mine;
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) s_wave[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int i = 0; i < kLeafThreads / 64; i++) {
+      const int v = s_wave[i];
+      s_wave[i]   = run;
+      run += v;
+    }
+    s_pre[n_parents] = run;
+  }
+  __syncthreads();
+  int run = s_wave[wave] + incl - mine;
+#pragma unroll
+  for (int u = 0; u < kPer; u++) {
+    const int j = threadIdx.x * kPer + u;
+    if (j < n_parents) s_pre[j] = run;
+    run += len[u];
+  }
+  __syncthreads();
+  const int total = s_pre[n_parents];
+  for (int t = threadIdx.x; t < total; t += kLeafThreads) {
+    // last segment whose prefix is <= t (empty runs share a prefix; the last of them holds t)
+    int lo = 0, hi = n_parents;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (s_pre[mid] <= t)
+        lo = mid;
+      else
+        hi = mid;
+    }
+    const int row = pos[s_lo[lo] + (t - s_pre[lo])].y;
+    int node      = level_first + lo;
+    const int ft  = feature[node];
+    if (ft != -1)
+      node = static_cast<int>(bins_t[ft * bins_stride + row]) <= split_bin[node] ? left_child(node) : right_child(node);
+    row_leaf[row] = node;
+  }
+}
+
 // pass 2: exclusive scan of the per-workgroup counts (single workgroup of 1024
 // threads; every thread owns a contiguous slice, slices are joined by a wave
 // scan and a scan over the 16 wave totals)
@@ -944,6 +1050,7 @@ struct Layout {
   int2* block_offsets;
   int2* totals;
   int2* seg_prefix;
+  int32_t* leaf_bounds;
   // histogram
   int32_t* tile_start;
   int4* tiles;
@@ -1013,6 +1120,7 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.block_offsets = ar.take<int2>(n_pblocks);
   L.totals        = ar.take<int2>(1);
   L.seg_prefix    = ar.take<int2>(level_nodes);
+  L.leaf_bounds   = max_depth >= 2 ? ar.take<int32_t>(kLeafBoundsEntries) : nullptr;
   L.tile_start    = ar.take<int32_t>(level_nodes + 1);
   // a tile holds at least 8 rows (two rows per pass, four passes); every node adds at most one partial tile
   L.tiles         = ar.take<int4>(N / 8 + level_nodes + 1);
@@ -1254,7 +1362,23 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   if (row_leaf != nullptr) {
     ProfScope ps(LBT_PROF_POSITIONS, stream);
     const bool bt = use_bins_t && max_depth >= 2;
-    if (bt && hs.bin_bytes == 2)
+    const int n_parents = static_cast<int>(int64_t(1) << (max_depth > 0 ? max_depth - 1 : 0));
+    const int n_windows = static_cast<int>((N + kLeafWindow - 1) / kLeafWindow);
+    const int64_t bound_entries = static_cast<int64_t>(n_parents) * (n_windows + 1);
+    if (bt && n_parents <= kLeafParents && bound_entries <= kLeafBoundsEntries) {
+      // positions of the last level: segments level_first .. level_first + n_parents - 1
+      const int level_first = static_cast<int>(level_begin(max_depth - 1));
+      leaf_window_bounds_kernel<<<blocks(bound_entries, kThreads), kThreads, 0, stream>>>(
+        L.pos[cur_pos], L.seg[cur_seg], n_parents, n_windows, L.leaf_bounds);
+      if (hs.bin_bytes == 2)
+        final_leaf_window_kernel<uint16_t><<<n_windows, kLeafThreads, 0, stream>>>(
+          L.pos[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint16_t*>(L.bins_t),
+          L.bins_t_stride, feature, L.split_bin, row_leaf);
+      else
+        final_leaf_window_kernel<uint8_t><<<n_windows, kLeafThreads, 0, stream>>>(
+          L.pos[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint8_t*>(L.bins_t),
+          L.bins_t_stride, feature, L.split_bin, row_leaf);
+    } else if (bt && hs.bin_bytes == 2)
       final_leaf_kernel<T, uint16_t><<<blocks(N, kThreads), kThreads, 0, stream>>>(
         L.pos[cur_pos], N, X, F, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, split,
         L.split_bin, max_nodes, row_leaf);

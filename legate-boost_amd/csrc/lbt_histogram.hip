@@ -656,8 +656,10 @@ __global__ void __launch_bounds__(kHistThreads)
     tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
     tz_words         = ((ri.bins_end | ri.zero_end) & 3) == 0;
   }
-  const int64_t r_begin = a.n_rows * chunk / a.n_chunks;
-  const int64_t r_end   = a.n_rows * (chunk + 1) / a.n_chunks;
+  // chunks start on multiples of 32 rows: with X itself aligned, the kilobyte a wave loads
+  // then begins on a cache line whatever the row length is
+  const int64_t r_begin = (a.n_rows * chunk / a.n_chunks) & ~int64_t(31);
+  const int64_t r_end   = chunk + 1 == a.n_chunks ? a.n_rows : (a.n_rows * (chunk + 1) / a.n_chunks) & ~int64_t(31);
   // Inside the chunk rows are numbered from 0 and addressed by 32-bit byte offsets (the host
   // keeps a chunk's rows times the widest row below 2^31 bytes), which advance by a uniform
   // step from pass to pass instead of being multiplied out per row.
@@ -1144,7 +1146,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     per_xcd          = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (b.n_rows / (hs.rpp * kUnroll) + 7) / 8));
     // the kernel addresses a chunk's rows with 32-bit byte offsets
     const int64_t widest = std::max<int64_t>(static_cast<int64_t>(b.F) * sizeof(T), hs.max_rec_stride);
-    while ((b.n_rows / (per_xcd * 8) + 2) * widest >= (int64_t(1) << 31)) per_xcd *= 2;
+    while ((b.n_rows / (per_xcd * 8) + 34) * widest >= (int64_t(1) << 31)) per_xcd *= 2;
     a.n_chunks       = static_cast<int>(per_xcd * 8);
     const unsigned grid = static_cast<unsigned>(per_xcd * 8 * hs.n_sgroups);
     int rc = LBT_OK;

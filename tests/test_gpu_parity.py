@@ -309,14 +309,16 @@ def test_log_loss_gradient_matches_oracle(k):
     assert np.isfinite(gu.cpu(g_g)).all() and (gu.cpu(h_g) >= 1e-8).all()
 
 
-@pytest.mark.parametrize("k", [1, 4])
-def test_row_leaf_prediction_update_equals_predict(k):
+# depth 13 / 14: the last level has 4096 / 8192 segments, either side of what the windowed leaf
+# kernel indexes; 600 split samples: two-byte bins; depth 1: no bin cache
+@pytest.mark.parametrize("k,depth,s", [(1, 6, 64), (4, 6, 64), (1, 13, 16), (1, 14, 16), (2, 5, 600), (1, 1, 64)])
+def test_row_leaf_prediction_update_equals_predict(k, depth, s):
     import gpu_util as gu
     import oracle_lib as orc
     from lbtree import ops
 
     X, g, h = _problem(60 + k, 30000, 9, k)
-    r = ops.build_tree(X, g, h, max_depth=6, split_samples=64, seed=3, row_leaf=True)
+    r = ops.build_tree(X, g, h, max_depth=depth, split_samples=s, seed=3, row_leaf=True)
     base = np.random.RandomState(1).normal(size=(30000, k))
     pred = torch.from_numpy(base.copy()).cuda()
     ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
