@@ -644,17 +644,31 @@ __global__ void __launch_bounds__(kHistThreads)
   const T cmax         = static_cast<T>(C - 1);
   const int pitch      = a.bin_stride[fb];
   BinT* const bin_base = binned + a.bin_base[fb];
-  // what this lane writes behind its own bins (byte offsets from its first bin)
+  // what this lane writes behind its own bins (byte offsets from its first bin). A record ends
+  // with zero padding and, for single-output trees, the row's gradient pair in its last 8
+  // bytes; where it can, the lane writes the record's last 16 bytes with one store, so that
+  // every record reaches memory as whole, aligned pieces.
   const int tg = a.bin_tail[fb + VEC - 1];
-  int tz_from = 0, tz_to = 0, tq = -1;
+  int tz_from = 0, tz_to = 0, tq = -1, t16 = 0;
   bool tz_words = false;
+  int tmode     = 0;  // 1: zeros, then the pair on its own; 2: own bins + pair in one store; 3: zeros, then [0, 0, pair]
   if (tg > 0) {
     const RecInfo ri = a.rec[tg - 1];
     const int my_off = static_cast<int>(a.bin_base[fb] * static_cast<int64_t>(sizeof(BinT)) - ri.base);
     tz_from          = ri.bins_end - my_off;
     tz_to            = ri.zero_end - my_off;
     tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
-    tz_words         = ((ri.bins_end | ri.zero_end) & 3) == 0;
+    tmode            = 1;
+    if (VEC * sizeof(BinT) == 4 && ri.q_off >= 0 && ri.q_off == ri.stride - 8) {
+      t16 = ri.stride - 16 - my_off;
+      if (t16 == 0 && ri.bins_end == my_off + 4) {
+        tmode = 2;
+      } else if (ri.bins_end <= ri.stride - 16) {
+        tmode = 3;
+        tz_to = t16;
+      }
+    }
+    tz_words = ((tz_from | tz_to) & 3) == 0;
   }
   // chunks start on multiples of 32 rows: with X itself aligned, the kilobyte a wave loads
   // then begins on a cache line whatever the row length is
@@ -743,20 +757,33 @@ __global__ void __launch_bounds__(kHistThreads)
         }
         unsigned char* tail = b_chunk + (b_off0 + u * b_step);
         BinT* bp            = reinterpret_cast<BinT*>(tail);
-        if constexpr (VEC == 4 && sizeof(BinT) == 1) {
-          *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
-                                             (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
-        } else {
+        if (tmode == 2) {
+          // VEC * sizeof(BinT) == 4: the lane's bins are one word
+          uint32_t mine = 0;
 #pragma unroll
-          for (int v = 0; v < VEC; v++) bp[v] = rel[v];
-        }
-        if (tg > 0) {
-          if (tz_words) {
-            for (int i = tz_from; i < tz_to; i += 4) *reinterpret_cast<uint32_t*>(tail + i) = 0u;
+          for (int v = 0; v < VEC; v++) mine |= static_cast<uint32_t>(rel[v]) << (8 * sizeof(BinT) * (v & 3));
+          *reinterpret_cast<uint4*>(tail) =
+            make_uint4(mine, 0u, static_cast<uint32_t>(q_c[u].x), static_cast<uint32_t>(q_c[u].y));
+        } else {
+          if constexpr (VEC == 4 && sizeof(BinT) == 1) {
+            *reinterpret_cast<uint32_t*>(bp) = static_cast<uint32_t>(rel[0]) | (static_cast<uint32_t>(rel[1]) << 8) |
+                                               (static_cast<uint32_t>(rel[2]) << 16) | (static_cast<uint32_t>(rel[3]) << 24);
           } else {
-            for (int i = tz_from; i < tz_to; i++) tail[i] = 0;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) bp[v] = rel[v];
           }
-          if (tq >= 0) *reinterpret_cast<int2*>(tail + tq) = q_c[u];
+          if (tmode != 0) {
+            if (tz_words) {
+              for (int i = tz_from; i < tz_to; i += 4) *reinterpret_cast<uint32_t*>(tail + i) = 0u;
+            } else {
+              for (int i = tz_from; i < tz_to; i++) tail[i] = 0;
+            }
+            if (tmode == 3)
+              *reinterpret_cast<uint4*>(tail + t16) =
+                make_uint4(0u, 0u, static_cast<uint32_t>(q_c[u].x), static_cast<uint32_t>(q_c[u].y));
+            else if (tq >= 0)
+              *reinterpret_cast<int2*>(tail + tq) = q_c[u];
+          }
         }
       }
     }
@@ -1368,15 +1395,12 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       const int chunk_end = (bins_end + chunk - 1) / chunk * chunk;
       RecInfo& ri         = rec[g];
       ri.bins_end         = bins_end;
-      if (hs.embed) {
-        ri.q_off    = (bins_end + 7) / 8 * 8;
-        ri.zero_end = ri.q_off;
-      } else {
-        ri.q_off    = -1;
-        ri.zero_end = chunk_end;
-      }
-      const int used = std::max(chunk_end, hs.embed ? ri.q_off + 8 : 0);
+      // bins, zeros up to the end of the record, the gradient pair (if embedded) in the last 8
+      // bytes: every byte of a record is written, so no cache line reaches memory in parts
+      const int used = std::max(chunk_end, hs.embed ? (bins_end + 7) / 8 * 8 + 8 : 0);
       ri.stride      = (used + 31) / 32 * 32;
+      ri.q_off       = hs.embed ? ri.stride - 8 : -1;
+      ri.zero_end    = hs.embed ? ri.q_off : ri.stride;
       hs.max_rec_stride = std::max<int64_t>(hs.max_rec_stride, ri.stride);
       ri.base        = at;
       for (int f = groups[g]; f < groups[g + 1]; f++) {
