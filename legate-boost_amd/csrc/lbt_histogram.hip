@@ -659,11 +659,11 @@ __global__ void __launch_bounds__(kHistThreads)
     tz_to            = ri.zero_end - my_off;
     tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
     tmode            = 1;
-    if (VEC * sizeof(BinT) == 4 && ri.q_off >= 0 && ri.q_off == ri.stride - 8) {
-      t16 = ri.stride - 16 - my_off;
+    if (VEC * sizeof(BinT) == 4 && ri.q_off >= 0 && ri.q_off == ri.size - 8) {
+      t16 = ri.size - 16 - my_off;
       if (t16 == 0 && ri.bins_end == my_off + 4) {
         tmode = 2;
-      } else if (ri.bins_end <= ri.stride - 16) {
+      } else if (ri.bins_end <= ri.size - 16) {
         tmode = 3;
         tz_to = t16;
       }
@@ -1387,8 +1387,11 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
     // record layout of every histogram group
     const int chunk = hs.bvec * hs.bin_bytes;  // bytes a lane of the histogram kernel loads
-    int64_t at      = 0;
+    // The records of a row lie side by side ([row][group]): the binning pass, whose lanes hold a
+    // whole row, then writes one contiguous piece per row, and the workgroups that read the
+    // groups of the same rows at the same time share the cache lines.
     rec.resize(hs.n_groups);
+    int pitch = 0;
     for (int g = 0; g < hs.n_groups; g++) {
       const int gs        = groups[g + 1] - groups[g];
       const int bins_end  = gs * hs.bin_bytes;
@@ -1398,18 +1401,23 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       // bins, zeros up to the end of the record, the gradient pair (if embedded) in the last 8
       // bytes: every byte of a record is written, so no cache line reaches memory in parts
       const int used = std::max(chunk_end, hs.embed ? (bins_end + 7) / 8 * 8 + 8 : 0);
-      ri.stride      = (used + 31) / 32 * 32;
-      ri.q_off       = hs.embed ? ri.stride - 8 : -1;
-      ri.zero_end    = hs.embed ? ri.q_off : ri.stride;
-      hs.max_rec_stride = std::max<int64_t>(hs.max_rec_stride, ri.stride);
-      ri.base        = at;
+      ri.size        = (used + 31) / 32 * 32;
+      ri.q_off       = hs.embed ? ri.size - 8 : -1;
+      ri.zero_end    = hs.embed ? ri.q_off : ri.size;
+      ri.base        = pitch;
+      pitch += ri.size;
+    }
+    hs.max_rec_stride = pitch;
+    for (int g = 0; g < hs.n_groups; g++) {
+      RecInfo& ri = rec[g];
+      ri.stride   = pitch;
       for (int f = groups[g]; f < groups[g + 1]; f++) {
-        base[f]   = at / hs.bin_bytes + (f - groups[g]);
-        stride[f] = ri.stride / hs.bin_bytes;
+        base[f]   = ri.base / hs.bin_bytes + (f - groups[g]);
+        stride[f] = pitch / hs.bin_bytes;
       }
       tail[groups[g + 1] - 1] = g + 1;
-      at += n_rows * ri.stride;
     }
+    const int64_t at = n_rows * static_cast<int64_t>(pitch);
     if (static_cast<size_t>(at) > hs.binned_capacity) {
       set_error("bin cache of %lld bytes exceeds the workspace share", static_cast<long long>(at));
       return LBT_ERR_WORKSPACE;

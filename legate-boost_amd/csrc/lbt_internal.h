@@ -281,7 +281,8 @@ struct LevelMeta {
 // bytes up to zero_end, and (single-output trees) the row's packed (grad, hess) pair at q_off.
 struct RecInfo {
   int64_t base;      // byte offset of row 0's record
-  int32_t stride;    // bytes between consecutive rows (multiple of 32)
+  int32_t stride;    // bytes between the records of consecutive rows (multiple of 32)
+  int32_t size;      // bytes of one record (multiple of 32)
   int32_t q_off;     // byte offset of the int2 (grad, hess) inside a record, or -1
   int32_t zero_end;  // bytes [bins_end, zero_end) of a record are zero
   int32_t bins_end;  // bytes of bins in a record
