@@ -396,12 +396,6 @@ __global__ void root_leaf_kernel(double* leaf, const I64Pair* node_sums, int K,
   }
 }
 
-// build_tree.cu:967-974
-__global__ void fill_positions_kernel(int2* pos, int64_t n)
-{
-  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
-  if (i < n) pos[i] = make_int2(0, static_cast<int>(i));
-}
 
 // ---------------------------------------------------------------------------
 // scan + sibling subtraction (build_tree.cu:597-668), one wave per
@@ -605,38 +599,75 @@ __global__ void proposals_to_double_kernel(const T* p, int n, double* out)
 // retired rows move to the front, then for each parent its left rows followed
 // by its right rows. Exclusive prefix counts of the "retired" and "left" flags
 // give every destination directly.
+//
+// The order is held as the list of row numbers alone. The rows of the level's
+// node j are the run seg[j] .. seg[j+1] of that list, the rows in front of
+// seg[0] have retired, so an index finds its node by its place among the
+// segment starts and the node field never travels through memory.
 
 constexpr int kPartItems = 8;
-constexpr int kPartBlock = kThreads * kPartItems;  // rows per workgroup
+constexpr int kPartBlock = kThreads * kPartItems;  // indices per workgroup ("slab")
+constexpr int kSegLds    = kPartBlock + 64;        // segment starts a workgroup keeps in the LDS
 
-// pass 1: classify each row (0 retired, 1 left, 2 right) and count per workgroup
-template <typename T>
-__global__ void __launch_bounds__(kThreads)
-  classify_kernel(const int2* pos, int64_t n, const T* X, int F, const int32_t* feature,
-                  const double* split, int max_nodes, uint8_t* code, int2* block_counts)
+// The segments that meet one slab: the one that holds its first index (known per slab,
+// block_seg) and the m that start inside it.
+struct SlabSegments {
+  int j0;       // segment of the slab's first index; -1: it lies among the retired rows
+  int m;        // segments j0+1 .. j0+m start inside the slab
+  bool in_lds;  // their starts are in the LDS (else they are read from seg)
+};
+
+// All threads of the workgroup call this; s_seg has kSegLds entries.
+__device__ inline SlabSegments load_slab_segments(const int32_t* __restrict__ seg, int n_parents,
+                                                  const int32_t* __restrict__ block_seg, int64_t base, int64_t n,
+                                                  int* s_seg)
 {
-  __shared__ int s_d[kThreads / 64];
-  __shared__ int s_l[kThreads / 64];
-  const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
-  int nd = 0, nl = 0;
-#pragma unroll
-  for (int u = 0; u < kPartItems; u++) {
-    int64_t i = base + u * kThreads + threadIdx.x;
-    if (i < n) {
-      int2 p = pos[i];
-      int c  = 0;
-      if (p.x >= 0 && p.x < max_nodes) {
-        int ft = feature[p.x];
-        if (ft != -1) {
-          double xv = static_cast<double>(X[static_cast<int64_t>(p.y) * F + ft]);
-          c         = xv <= split[p.x] ? 1 : 2;
-        }
-      }
-      code[i] = static_cast<uint8_t>(c);
-      nd += c == 0;
-      nl += c == 1;
+  SlabSegments ss;
+  ss.j0         = block_seg[blockIdx.x];
+  const int end = static_cast<int>(base + kPartBlock < n ? base + kPartBlock : n);
+  ss.m          = 0;
+  // the starts ascend, so those inside the slab are a prefix of seg[j0+1 ..]
+  for (int k = 0;; k += kThreads) {
+    const int64_t idx = static_cast<int64_t>(ss.j0) + 1 + k + threadIdx.x;
+    const int v       = idx < n_parents ? seg[idx] : 2147483647;
+    const bool inside = v < end;
+    if (inside && k + static_cast<int>(threadIdx.x) < kSegLds) s_seg[k + threadIdx.x] = v;
+    const int cnt = __syncthreads_count(inside);
+    ss.m += cnt;
+    if (cnt < kThreads) break;
+  }
+  ss.in_lds = ss.m <= kSegLds;
+  return ss;
+}
+
+// Segment of index i of the slab (-1: retired): j0 plus the number of starts at or below i.
+// Of several segments that start at the same index the last one is not empty.
+__device__ inline int segment_of(const SlabSegments& ss, const int* s_seg, const int32_t* __restrict__ seg, int i)
+{
+  int lo = 0, hi = ss.m;
+  if (ss.in_lds) {
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (s_seg[mid] <= i)
+        lo = mid + 1;
+      else
+        hi = mid;
+    }
+  } else {
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (seg[ss.j0 + 1 + mid] <= i)
+        lo = mid + 1;
+      else
+        hi = mid;
     }
   }
+  return ss.j0 + lo;
+}
+
+// adds up the per-thread counts of a workgroup and stores them for the scan
+__device__ inline void store_block_counts(int nd, int nl, int* s_d, int* s_l, int2* block_counts)
+{
   for (int off = 32; off >= 1; off >>= 1) {
     nd += __shfl_down(nd, off, 64);
     nl += __shfl_down(nl, off, 64);
@@ -653,6 +684,41 @@ __global__ void __launch_bounds__(kThreads)
     }
     block_counts[blockIdx.x] = make_int2(nd, nl);
   }
+}
+
+// pass 1: classify each row (0 retired, 1 left, 2 right) and count per workgroup
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+  classify_kernel(const int32_t* __restrict__ rows, int64_t n, const int32_t* __restrict__ seg,
+                  const int32_t* __restrict__ block_seg, int n_parents, int level_first, const T* X, int F,
+                  const int32_t* feature, const double* split, uint8_t* code, int2* block_counts)
+{
+  __shared__ int s_seg[kSegLds];
+  __shared__ int s_d[kThreads / 64];
+  __shared__ int s_l[kThreads / 64];
+  const int64_t base    = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  const SlabSegments ss = load_slab_segments(seg, n_parents, block_seg, base, n, s_seg);
+  int nd = 0, nl = 0;
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    if (i < n) {
+      const int j = segment_of(ss, s_seg, seg, static_cast<int>(i));
+      int c       = 0;
+      if (j >= 0) {
+        const int node = level_first + j;
+        const int ft   = feature[node];
+        if (ft != -1) {
+          const double xv = static_cast<double>(X[static_cast<int64_t>(rows[i]) * F + ft]);
+          c               = xv <= split[node] ? 1 : 2;
+        }
+      }
+      code[i] = static_cast<uint8_t>(c);
+      nd += c == 0;
+      nl += c == 1;
+    }
+  }
+  store_block_counts(nd, nl, s_d, s_l, block_counts);
 }
 
 constexpr int kTransRows = 128;  // the feature-major bins are padded to whole groups of this many rows
@@ -662,70 +728,81 @@ constexpr int kTransRows = 128;  // the feature-major bins are padded to whole g
 // decides the side and consecutive rows of a node read consecutive bytes.
 template <typename BinT>
 __global__ void __launch_bounds__(kThreads)
-  classify_bins_kernel(const int2* pos, int64_t n, const BinT* bins_t, int64_t bins_stride,
-                       const int32_t* feature, const int32_t* split_bin, int max_nodes, uint8_t* code,
-                       int2* block_counts)
+  classify_bins_kernel(const int32_t* __restrict__ rows, int64_t n, const int32_t* __restrict__ seg,
+                       const int32_t* __restrict__ block_seg, int n_parents, int level_first,
+                       const BinT* __restrict__ bins_t, int64_t bins_stride, const int32_t* feature,
+                       const int32_t* split_bin, uint8_t* code, int2* block_counts)
 {
+  __shared__ int s_seg[kSegLds];
   __shared__ int s_d[kThreads / 64];
   __shared__ int s_l[kThreads / 64];
   const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  // the row numbers are requested before the slab's segments, which they do not depend on
+  int row[kPartItems];
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    row[u]          = i < n ? rows[i] : 0;
+  }
+  const SlabSegments ss = load_slab_segments(seg, n_parents, block_seg, base, n, s_seg);
+  int node[kPartItems], ft[kPartItems], sb[kPartItems];
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    const int j     = i < n ? segment_of(ss, s_seg, seg, static_cast<int>(i)) : -1;
+    node[u]         = j >= 0 ? level_first + j : -1;
+    ft[u]           = j >= 0 ? feature[node[u]] : -1;
+    sb[u]           = j >= 0 ? split_bin[node[u]] : 0;
+  }
+  int bin[kPartItems];
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++)
+    bin[u] = ft[u] != -1 ? static_cast<int>(bins_t[ft[u] * bins_stride + row[u]]) : 0;
   int nd = 0, nl = 0;
 #pragma unroll
   for (int u = 0; u < kPartItems; u++) {
-    int64_t i = base + u * kThreads + threadIdx.x;
+    const int64_t i = base + u * kThreads + threadIdx.x;
     if (i < n) {
-      int2 p = pos[i];
-      int c  = 0;
-      if (p.x >= 0 && p.x < max_nodes) {
-        int ft = feature[p.x];
-        if (ft != -1) c = static_cast<int>(bins_t[ft * bins_stride + p.y]) <= split_bin[p.x] ? 1 : 2;
-      }
-      code[i] = static_cast<uint8_t>(c);
+      const int c = ft[u] == -1 ? 0 : (bin[u] <= sb[u] ? 1 : 2);
+      code[i]     = static_cast<uint8_t>(c);
       nd += c == 0;
       nl += c == 1;
     }
   }
-  for (int off = 32; off >= 1; off >>= 1) {
-    nd += __shfl_down(nd, off, 64);
-    nl += __shfl_down(nl, off, 64);
-  }
-  if ((threadIdx.x & 63) == 0) {
-    s_d[threadIdx.x >> 6] = nd;
-    s_l[threadIdx.x >> 6] = nl;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < kThreads / 64; w++) {
-      nd += s_d[w];
-      nl += s_l[w];
-    }
-    block_counts[blockIdx.x] = make_int2(nd, nl);
-  }
+  store_block_counts(nd, nl, s_d, s_l, block_counts);
 }
 
 // Leaf of every row that is still in a node after the last level: the node itself if it
 // did not split, else the child the row falls into.
 template <typename T, typename BinT>
 __global__ void __launch_bounds__(kThreads)
-  final_leaf_kernel(const int2* pos, int64_t n, const T* X, int F, const BinT* bins_t, int64_t bins_stride,
-                    const int32_t* feature, const double* split, const int32_t* split_bin, int max_nodes,
-                    int32_t* row_leaf)
+  final_leaf_kernel(const int32_t* __restrict__ rows, int64_t n, const int32_t* __restrict__ seg,
+                    const int32_t* __restrict__ block_seg, int n_parents, int level_first, const T* X, int F,
+                    const BinT* bins_t, int64_t bins_stride, const int32_t* feature, const double* split,
+                    const int32_t* split_bin, int32_t* row_leaf)
 {
-  int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
-  if (i >= n) return;
-  int2 p = pos[i];
-  if (p.x < 0 || p.x >= max_nodes) return;  // retired earlier: recorded when it retired
-  int node = p.x;
-  int ft   = feature[node];
-  if (ft != -1) {
-    bool left;
-    if (bins_t != nullptr)
-      left = static_cast<int>(bins_t[ft * bins_stride + p.y]) <= split_bin[node];
-    else
-      left = static_cast<double>(X[static_cast<int64_t>(p.y) * F + ft]) <= split[node];
-    node = left ? left_child(node) : right_child(node);
+  __shared__ int s_seg[kSegLds];
+  const int64_t base    = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  const SlabSegments ss = load_slab_segments(seg, n_parents, block_seg, base, n, s_seg);
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    if (i >= n) continue;
+    const int j = segment_of(ss, s_seg, seg, static_cast<int>(i));
+    if (j < 0) continue;  // retired earlier: recorded when it retired
+    int node      = level_first + j;
+    const int row = rows[i];
+    const int ft  = feature[node];
+    if (ft != -1) {
+      bool left;
+      if (bins_t != nullptr)
+        left = static_cast<int>(bins_t[ft * bins_stride + row]) <= split_bin[node];
+      else
+        left = static_cast<double>(X[static_cast<int64_t>(row) * F + ft]) <= split[node];
+      node = left ? left_child(node) : right_child(node);
+    }
+    row_leaf[row] = node;
   }
-  row_leaf[p.y] = node;
 }
 
 // The same result, written window by window of the row space. The rows of a node ascend
@@ -740,7 +817,8 @@ constexpr int64_t kLeafBoundsEntries = int64_t(1) << 20;
 
 // bounds[j * (n_windows + 1) + w] = first index of segment j whose row is >= w * kLeafWindow
 __global__ void __launch_bounds__(kThreads)
-  leaf_window_bounds_kernel(const int2* pos, const int32_t* seg, int n_parents, int n_windows, int32_t* bounds)
+  leaf_window_bounds_kernel(const int32_t* __restrict__ rows, const int32_t* seg, int n_parents, int n_windows,
+                            int32_t* bounds)
 {
   const int64_t t = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
   if (t >= static_cast<int64_t>(n_parents) * (n_windows + 1)) return;
@@ -753,7 +831,7 @@ __global__ void __launch_bounds__(kThreads)
     const int64_t first = static_cast<int64_t>(w) * kLeafWindow;
     while (lo < hi) {
       const int mid = lo + ((hi - lo) >> 1);
-      if (pos[mid].y < first)
+      if (rows[mid] < first)
         lo = mid + 1;
       else
         hi = mid;
@@ -764,8 +842,8 @@ __global__ void __launch_bounds__(kThreads)
 
 template <typename BinT>
 __global__ void __launch_bounds__(kLeafThreads)
-  final_leaf_window_kernel(const int2* pos, const int32_t* bounds, int n_parents, int n_windows, int level_first,
-                           const BinT* bins_t, int64_t bins_stride, const int32_t* feature,
+  final_leaf_window_kernel(const int32_t* __restrict__ rows, const int32_t* bounds, int n_parents, int n_windows,
+                           int level_first, const BinT* bins_t, int64_t bins_stride, const int32_t* feature,
                            const int32_t* split_bin, int32_t* row_leaf)
 {
   __shared__ int s_lo[kLeafParents];
@@ -825,7 +903,7 @@ __global__ void __launch_bounds__(kLeafThreads)
       else
         hi = mid;
     }
-    const int row = pos[s_lo[lo] + (t - s_pre[lo])].y;
+    const int row = rows[s_lo[lo] + (t - s_pre[lo])];
     int node      = level_first + lo;
     const int ft  = feature[node];
     if (ft != -1)
@@ -897,27 +975,38 @@ __device__ inline int2 prefix_at(int s, int64_t n, const uint8_t* code, const in
   return make_int2(off.x + nd, off.y + nl);
 }
 
-// pass 3: one wave per parent j: prefix counts at its segment start, and the
-// segment starts of its two children in the next level.
+// pass 3: one wave per parent j: prefix counts at its segment start, the segment starts
+// of its two children in the next level, and for every slab of the next level's order
+// that begins inside one of these children the child's number (what load_slab_segments
+// starts from). The wave of parent 0 also marks the slabs that begin among the retired rows.
 __global__ void __launch_bounds__(kThreads)
   child_segments_kernel(const int32_t* seg, int n_parents, int64_t n, const uint8_t* code,
                         const int2* block_offsets, const int2* totals, int2* seg_prefix,
-                        int32_t* seg_next)
+                        int32_t* seg_next, int32_t* block_seg_next)
 {
   const int lane = threadIdx.x & 63;
   const int j    = static_cast<int>((blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x) >> 6);
   if (j >= n_parents) return;
-  int s0 = seg[j], s1 = seg[j + 1];
-  int2 p0 = prefix_at(s0, n, code, block_offsets, totals, lane);
-  int2 p1 = prefix_at(s1, n, code, block_offsets, totals, lane);
+  const int s0 = seg[j], s1 = seg[j + 1];
+  const int2 p0 = prefix_at(s0, n, code, block_offsets, totals, lane);
+  const int2 p1 = prefix_at(s1, n, code, block_offsets, totals, lane);
+  const int total_dead = totals->x;
+  const int left  = total_dead + (s0 - p0.x);          // start of the left child's run
+  const int right = left + (p1.y - p0.y);              // start of the right child's run
+  const int end   = left + (s1 - s0) - (p1.x - p0.x);  // end of the right child's run
   if (lane == 0) {
-    int total_dead      = totals->x;
-    int base            = total_dead + (s0 - p0.x);
     seg_prefix[j]       = p0;
-    seg_next[2 * j]     = base;
-    seg_next[2 * j + 1] = base + (p1.y - p0.y);
+    seg_next[2 * j]     = left;
+    seg_next[2 * j + 1] = right;
     if (j == n_parents - 1) seg_next[2 * n_parents] = static_cast<int32_t>(n);
   }
+  auto mark = [&](int from, int to, int value) {
+    for (int64_t b = (static_cast<int64_t>(from) + kPartBlock - 1) / kPartBlock + lane; b * kPartBlock < to; b += 64)
+      block_seg_next[b] = value;
+  };
+  if (j == 0) mark(0, total_dead, -1);
+  mark(left, right, 2 * j);
+  mark(right, end, 2 * j + 1);
 }
 
 // number of set bits of a 64-bit wave mask below the calling lane
@@ -927,29 +1016,53 @@ __device__ inline int prefix_popc(unsigned long long mask)
                                    __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0));
 }
 
-// pass 4: scatter every pair to its place in the next level's order. Rows are
+// pass 4: scatter every row to its place in the next level's order. Rows are
 // taken in slabs of one workgroup width (coalesced); inside a slab the ranks
 // come from wave ballots, across waves and slabs from a 32-entry scan.
 __global__ void __launch_bounds__(kThreads)
-  scatter_kernel(const int2* pos, int64_t n, const uint8_t* code, const int2* block_offsets,
-                 const int32_t* seg, const int2* seg_prefix, const int32_t* seg_next,
-                 int level_first, int n_parents, int2* pos_out, int32_t* row_leaf)
+  scatter_kernel(const int32_t* __restrict__ rows, int64_t n, const uint8_t* code, const int2* block_offsets,
+                 const int32_t* __restrict__ seg, const int32_t* __restrict__ block_seg, const int2* seg_prefix,
+                 const int32_t* seg_next, int level_first, int n_parents, int32_t* rows_out, int32_t* row_leaf)
 {
   constexpr int kWaves = kThreads / 64;
+  __shared__ int s_seg[kSegLds];
   __shared__ int s_cnt[kPartItems * kWaves];  // retired << 16 | left, in row order
   const int64_t base = blockIdx.x * static_cast<int64_t>(kPartBlock);
-  const int wave = threadIdx.x >> 6;
-  int2 p[kPartItems];
+  const int wave     = threadIdx.x >> 6;
+  int row[kPartItems];
   int c[kPartItems];
   int below_d[kPartItems], below_l[kPartItems];
+  // rows and codes are requested before the slab's segments, which they do not depend on
 #pragma unroll
   for (int u = 0; u < kPartItems; u++) {
     int64_t i = base + u * kThreads + threadIdx.x;
     c[u]      = 3;
+    row[u]    = 0;
     if (i < n) {
-      p[u] = pos[i];
-      c[u] = code[i];
+      row[u] = rows[i];
+      c[u]   = code[i];
     }
+  }
+  const SlabSegments ss = load_slab_segments(seg, n_parents, block_seg, base, n, s_seg);
+  const int2 boff       = block_offsets[blockIdx.x];
+  // Per row: its segment and what its destination is counted from. A left row goes to
+  // seg_next[2j] + (left rows of the segment before it), a right row to seg_next[2j+1] + (right
+  // rows of the segment before it); both counts are differences of prefix counts, whose
+  // segment-start part is known here already.
+  int seg_j[kPartItems], dbase[kPartItems];
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    seg_j[u]        = i < n ? segment_of(ss, s_seg, seg, static_cast<int>(i)) : -1;
+    dbase[u]        = 0;
+    if (c[u] == 1 || c[u] == 2) {
+      const int j   = seg_j[u];
+      const int2 sp = seg_prefix[j];
+      dbase[u]      = c[u] == 1 ? seg_next[2 * j] - sp.y : seg_next[2 * j + 1] - (seg[j] - sp.x - sp.y);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
     unsigned long long md = __ballot(c[u] == 0);
     unsigned long long ml = __ballot(c[u] == 1);
     below_d[u]            = prefix_popc(md);
@@ -957,16 +1070,19 @@ __global__ void __launch_bounds__(kThreads)
     if ((threadIdx.x & 63) == 0) s_cnt[u * kWaves + wave] = (__popcll(md) << 16) | __popcll(ml);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int i = 0; i < kPartItems * kWaves; i++) {
-      int v    = s_cnt[i];
-      s_cnt[i] = run;
-      run += v;
+  // exclusive scan of the kPartItems * kWaves = 32 counts by one wave
+  static_assert(kPartItems * kWaves <= 64, "one wave scans the slab's counts");
+  if (wave == 0) {
+    const int lane = threadIdx.x;
+    const int v    = lane < kPartItems * kWaves ? s_cnt[lane] : 0;
+    int incl       = v;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int o = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += o;
     }
+    if (lane < kPartItems * kWaves) s_cnt[lane] = incl - v;
   }
   __syncthreads();
-  const int2 boff = block_offsets[blockIdx.x];
 #pragma unroll
   for (int u = 0; u < kPartItems; u++) {
     int64_t i = base + u * kThreads + threadIdx.x;
@@ -974,36 +1090,48 @@ __global__ void __launch_bounds__(kThreads)
       const int excl = s_cnt[u * kWaves + wave];
       const int D    = boff.x + (excl >> 16) + below_d[u];
       const int L    = boff.y + (excl & 0xffff) + below_l[u];
-      int dest, new_node;
+      int dest;
       if (c[u] == 0) {
-        dest     = D;
-        new_node = -1;
+        dest = D;
         // a row that retires now sits in a leaf: remember which
-        if (row_leaf != nullptr && p[u].x >= 0) row_leaf[p[u].y] = p[u].x;
+        if (row_leaf != nullptr && seg_j[u] >= 0) row_leaf[row[u]] = level_first + seg_j[u];
+      } else if (c[u] == 1) {
+        dest = dbase[u] + L;
       } else {
-        const int j   = p[u].x - level_first;
-        const int s0  = seg[j];
-        const int2 sp = seg_prefix[j];
-        if (c[u] == 1) {
-          dest     = seg_next[2 * j] + (L - sp.y);
-          new_node = left_child(p[u].x);
-        } else {
-          const int R  = static_cast<int>(i) - D - L;
-          const int R0 = s0 - sp.x - sp.y;
-          dest         = seg_next[2 * j + 1] + (R - R0);
-          new_node     = right_child(p[u].x);
-        }
+        dest = dbase[u] + (static_cast<int>(i) - D - L);
       }
-      pos_out[dest] = make_int2(new_node, p[u].y);
+      rows_out[dest] = row[u];
     }
   }
 }
 
-__global__ void init_seg_kernel(int32_t* seg, int32_t n)
+// The reference's (node, row) pairs, for the observation points: node of the level that the
+// order belongs to, -1 for retired rows.
+__global__ void __launch_bounds__(kThreads)
+  expand_positions_kernel(const int32_t* __restrict__ rows, int64_t n, const int32_t* __restrict__ seg,
+                          const int32_t* __restrict__ block_seg, int n_parents, int level_first, int2* out)
 {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
+  __shared__ int s_seg[kSegLds];
+  const int64_t base    = blockIdx.x * static_cast<int64_t>(kPartBlock);
+  const SlabSegments ss = load_slab_segments(seg, n_parents, block_seg, base, n, s_seg);
+#pragma unroll
+  for (int u = 0; u < kPartItems; u++) {
+    const int64_t i = base + u * kThreads + threadIdx.x;
+    if (i >= n) continue;
+    const int j = segment_of(ss, s_seg, seg, static_cast<int>(i));
+    out[i]      = make_int2(j >= 0 ? level_first + j : -1, rows[i]);
+  }
+}
+
+// build_tree.cu:967-974: every row starts in the root
+__global__ void fill_positions_kernel(int32_t* rows, int64_t n, int32_t* seg, int32_t* block_seg, int64_t n_slabs)
+{
+  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i < n) rows[i] = static_cast<int32_t>(i);
+  if (i < n_slabs) block_seg[i] = 0;
+  if (i == 0) {
     seg[0] = 0;
-    seg[1] = n;
+    seg[1] = static_cast<int32_t>(n);
   }
 }
 
@@ -1039,9 +1167,10 @@ struct Layout {
   double* part_a[2];
   double* part_b[2];
   int2* qgh;
-  // positions
-  int2* pos[2];
+  // positions: row numbers in node order, segment starts, first segment of every slab
+  int32_t* rows[2];
   int32_t* seg[2];
+  int32_t* block_seg[2];
   uint8_t* code;
   int32_t* split_bin;
   void* bins_t;
@@ -1105,10 +1234,12 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
     n_chunks    = (n_chunks + 4095) / 4096;
   }
   L.qgh    = ar.take<int2>(N * K);
-  L.pos[0] = ar.take<int2>(N);
-  L.pos[1] = ar.take<int2>(N);
-  L.seg[0] = ar.take<int32_t>(level_nodes + 1);
-  L.seg[1] = ar.take<int32_t>(level_nodes + 1);
+  L.rows[0] = ar.take<int32_t>(N);
+  L.rows[1] = ar.take<int32_t>(N);
+  L.seg[0]  = ar.take<int32_t>(level_nodes + 1);
+  L.seg[1]  = ar.take<int32_t>(level_nodes + 1);
+  L.block_seg[0] = ar.take<int32_t>((N + kPartBlock - 1) / kPartBlock);
+  L.block_seg[1] = ar.take<int32_t>((N + kPartBlock - 1) / kPartBlock);
   L.code   = ar.take<uint8_t>(N);
   L.split_bin = ar.take<int32_t>(max_nodes);
   // feature-major bins for the position update (needs the bin cache)
@@ -1217,8 +1348,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   LBT_HIP(hipMemcpyAsync(h_qstats, L.qstats, sizeof(h_qstats), hipMemcpyDeviceToHost, stream));
 
   // ---- positions and histogram cache (TreeBuilder ctor, build_tree.cu:997-1017)
-  fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.pos[0], N);
-  init_seg_kernel<<<1, 64, 0, stream>>>(L.seg[0], static_cast<int32_t>(N));
+  fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.rows[0], N, L.seg[0], L.block_seg[0],
+                                                                       (N + kPartBlock - 1) / kPartBlock);
   static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
   if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
 
@@ -1286,11 +1417,12 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   int32_t* row_leaf     = taps ? taps->row_leaf : nullptr;
   const int n_chunks = (B + kSplitChunk - 1) / kSplitChunk;
   for (int depth = 0; depth < max_depth; depth++) {
-    if (taps && taps->positions_per_level)
-      LBT_HIP(hipMemcpyAsync(taps->positions_per_level + static_cast<size_t>(depth) * N * 2, L.pos[cur_pos],
-                             sizeof(int2) * N, hipMemcpyDeviceToDevice, stream));
     const int64_t nodes_in_level = int64_t(1) << depth;
     const int level_first        = static_cast<int>(level_begin(depth));
+    if (taps && taps->positions_per_level)
+      expand_positions_kernel<<<blocks(N, kPartBlock), kThreads, 0, stream>>>(
+        L.rows[cur_pos], N, L.seg[cur_seg], L.block_seg[cur_seg], static_cast<int>(nodes_in_level), level_first,
+        reinterpret_cast<int2*>(taps->positions_per_level) + static_cast<size_t>(depth) * N);
     int64_t num_batches          = 1;
     if (nodes_in_level > max_batch_size) num_batches = (nodes_in_level + max_batch_size - 1) / max_batch_size;
     for (int64_t bi = 0; bi < num_batches; bi++) {
@@ -1309,7 +1441,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       const int n_nodes = j1 - j0;
       {
         HistBatch hb;
-        hb.X = X; hb.F = F; hb.qgh = L.qgh; hb.K = K; hb.positions = L.pos[cur_pos]; hb.seg = L.seg[cur_seg];
+        hb.X = X; hb.F = F; hb.qgh = L.qgh; hb.K = K; hb.rows = L.rows[cur_pos]; hb.seg = L.seg[cur_seg];
         hb.j0 = j0; hb.n_nodes = n_nodes; hb.level_first = level_first; hb.proposals = L.proposals;
         hb.row_pointers = L.row_pointers; hb.bin_feature = L.bin_feature; hb.hist = hv; hb.qstats = L.qstats; hb.node_sums = L.node_sums;
         hb.level_total = L.level_totals + depth; hb.n_rows = N;
@@ -1334,26 +1466,30 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       }
     }
     if (depth < max_depth - 1) {
-      ProfScope ps(LBT_PROF_POSITIONS, stream, static_cast<double>(N) * (8 + 8 + 2 + 64));
-      const unsigned nb = blocks(N, kPartBlock);
+      ProfScope ps(LBT_PROF_POSITIONS, stream, static_cast<double>(N) * (4 + 4 + 2 + 64));
+      const unsigned nb   = blocks(N, kPartBlock);
+      const int n_parents = static_cast<int>(nodes_in_level);
+      const int32_t* rows = L.rows[cur_pos];
+      const int32_t* seg  = L.seg[cur_seg];
+      const int32_t* bseg = L.block_seg[cur_seg];
       if (use_bins_t && hs.bin_bytes == 1)
         classify_bins_kernel<uint8_t><<<nb, kThreads, 0, stream>>>(
-          L.pos[cur_pos], N, static_cast<const uint8_t*>(L.bins_t), L.bins_t_stride, feature, L.split_bin,
-          max_nodes, L.code, L.block_counts);
+          rows, N, seg, bseg, n_parents, level_first, static_cast<const uint8_t*>(L.bins_t), L.bins_t_stride, feature,
+          L.split_bin, L.code, L.block_counts);
       else if (use_bins_t)
         classify_bins_kernel<uint16_t><<<nb, kThreads, 0, stream>>>(
-          L.pos[cur_pos], N, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, L.split_bin,
-          max_nodes, L.code, L.block_counts);
+          rows, N, seg, bseg, n_parents, level_first, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature,
+          L.split_bin, L.code, L.block_counts);
       else
-        classify_kernel<T><<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, X, F, feature, split, max_nodes, L.code,
-                                                        L.block_counts);
+        classify_kernel<T><<<nb, kThreads, 0, stream>>>(rows, N, seg, bseg, n_parents, level_first, X, F, feature, split,
+                                                        L.code, L.block_counts);
       scan_block_counts_kernel<<<1, kScanThreads, 0, stream>>>(L.block_counts, nb, L.block_offsets, L.totals);
-      const int n_parents = static_cast<int>(nodes_in_level);
       child_segments_kernel<<<blocks(static_cast<int64_t>(n_parents) * 64, kThreads), kThreads, 0, stream>>>(
-        L.seg[cur_seg], n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[cur_seg ^ 1]);
-      scatter_kernel<<<nb, kThreads, 0, stream>>>(L.pos[cur_pos], N, L.code, L.block_offsets, L.seg[cur_seg],
-                                                  L.seg_prefix, L.seg[cur_seg ^ 1], level_first, n_parents,
-                                                  L.pos[cur_pos ^ 1], row_leaf);
+        seg, n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[cur_seg ^ 1],
+        L.block_seg[cur_seg ^ 1]);
+      scatter_kernel<<<nb, kThreads, 0, stream>>>(rows, N, L.code, L.block_offsets, seg, bseg, L.seg_prefix,
+                                                  L.seg[cur_seg ^ 1], level_first, n_parents, L.rows[cur_pos ^ 1],
+                                                  row_leaf);
       cur_pos ^= 1;
       cur_seg ^= 1;
     }
@@ -1365,27 +1501,27 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     const int n_parents = static_cast<int>(int64_t(1) << (max_depth > 0 ? max_depth - 1 : 0));
     const int n_windows = static_cast<int>((N + kLeafWindow - 1) / kLeafWindow);
     const int64_t bound_entries = static_cast<int64_t>(n_parents) * (n_windows + 1);
+    // the order of the last level: segments level_first .. level_first + n_parents - 1
+    const int level_first = static_cast<int>(level_begin(max_depth > 0 ? max_depth - 1 : 0));
     if (bt && n_parents <= kLeafParents && bound_entries <= kLeafBoundsEntries) {
-      // positions of the last level: segments level_first .. level_first + n_parents - 1
-      const int level_first = static_cast<int>(level_begin(max_depth - 1));
       leaf_window_bounds_kernel<<<blocks(bound_entries, kThreads), kThreads, 0, stream>>>(
-        L.pos[cur_pos], L.seg[cur_seg], n_parents, n_windows, L.leaf_bounds);
+        L.rows[cur_pos], L.seg[cur_seg], n_parents, n_windows, L.leaf_bounds);
       if (hs.bin_bytes == 2)
         final_leaf_window_kernel<uint16_t><<<n_windows, kLeafThreads, 0, stream>>>(
-          L.pos[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint16_t*>(L.bins_t),
+          L.rows[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint16_t*>(L.bins_t),
           L.bins_t_stride, feature, L.split_bin, row_leaf);
       else
         final_leaf_window_kernel<uint8_t><<<n_windows, kLeafThreads, 0, stream>>>(
-          L.pos[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint8_t*>(L.bins_t),
+          L.rows[cur_pos], L.leaf_bounds, n_parents, n_windows, level_first, static_cast<const uint8_t*>(L.bins_t),
           L.bins_t_stride, feature, L.split_bin, row_leaf);
     } else if (bt && hs.bin_bytes == 2)
-      final_leaf_kernel<T, uint16_t><<<blocks(N, kThreads), kThreads, 0, stream>>>(
-        L.pos[cur_pos], N, X, F, static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, split,
-        L.split_bin, max_nodes, row_leaf);
+      final_leaf_kernel<T, uint16_t><<<blocks(N, kPartBlock), kThreads, 0, stream>>>(
+        L.rows[cur_pos], N, L.seg[cur_seg], L.block_seg[cur_seg], n_parents, level_first, X, F,
+        static_cast<const uint16_t*>(L.bins_t), L.bins_t_stride, feature, split, L.split_bin, row_leaf);
     else
-      final_leaf_kernel<T, uint8_t><<<blocks(N, kThreads), kThreads, 0, stream>>>(
-        L.pos[cur_pos], N, X, F, bt ? static_cast<const uint8_t*>(L.bins_t) : nullptr, L.bins_t_stride, feature,
-        split, L.split_bin, max_nodes, row_leaf);
+      final_leaf_kernel<T, uint8_t><<<blocks(N, kPartBlock), kThreads, 0, stream>>>(
+        L.rows[cur_pos], N, L.seg[cur_seg], L.block_seg[cur_seg], n_parents, level_first, X, F,
+        bt ? static_cast<const uint8_t*>(L.bins_t) : nullptr, L.bins_t_stride, feature, split, L.split_bin, row_leaf);
   }
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
@@ -1411,8 +1547,12 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       LBT_HIP(hipMemcpyAsync(taps->quantised, L.qgh, sizeof(int2) * N * K, hipMemcpyDeviceToDevice, stream));
     if (taps->node_sums)
       LBT_HIP(hipMemcpyAsync(taps->node_sums, L.node_sums, sizeof(I64Pair) * max_nodes * K, hipMemcpyDeviceToDevice, stream));
-    if (taps->positions)
-      LBT_HIP(hipMemcpyAsync(taps->positions, L.pos[cur_pos], sizeof(int2) * N, hipMemcpyDeviceToDevice, stream));
+    if (taps->positions) {
+      const int last = max_depth > 0 ? max_depth - 1 : 0;
+      expand_positions_kernel<<<blocks(N, kPartBlock), kThreads, 0, stream>>>(
+        L.rows[cur_pos], N, L.seg[cur_seg], L.block_seg[cur_seg], static_cast<int>(int64_t(1) << last),
+        static_cast<int>(level_begin(last)), reinterpret_cast<int2*>(taps->positions));
+    }
     if (taps->histogram) {
       int64_t nodes = taps->hist_node_end - taps->hist_node_begin;
       int64_t need  = nodes * K * B * 2;

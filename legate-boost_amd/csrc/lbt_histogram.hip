@@ -246,7 +246,7 @@ struct TileWalk {
 // the kernel touches them and fetch the uniform ones through the scalar cache;
 // vector loads here would force waits that also drain the prefetched row data.
 #define LBT_WALK_PARAMS                                                                 \
-  const int2* __restrict__ positions, const int4* __restrict__ tiles,                   \
+  const int32_t* __restrict__ positions, const int4* __restrict__ tiles,                   \
     const LevelMeta* __restrict__ meta, const unsigned long long* __restrict__ qstats
 
 struct Tile {
@@ -437,7 +437,7 @@ __global__ void __launch_bounds__(kHistThreads)
       if constexpr (kIdentityRows)
         row[u] = ok ? rr : t.r0;
       else
-        row[u] = positions[ok ? rr : t.r0].y;
+        row[u] = positions[ok ? rr : t.r0];
       valid |= ok ? (1u << u) : 0u;
     }
     return valid;
@@ -915,7 +915,7 @@ __global__ void __launch_bounds__(kHistThreads)
       if constexpr (kRoot)
         row[u] = ok ? rr : t.r0;  // the order is still the identity: sorted index == row
       else
-        row[u] = positions[ok ? rr : t.r0].y;
+        row[u] = positions[ok ? rr : t.r0];
       valid |= ok ? (1u << u) : 0u;
     }
     return valid;
@@ -1069,7 +1069,7 @@ int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a,
   static bool attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(histogram_kernel<T, VEC, kIdentityRows>, kLdsBudget, attr_set));
   histogram_kernel<T, VEC, kIdentityRows><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
-    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const T*>(b.X), b.qgh);
+    a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const T*>(b.X), b.qgh);
   return LBT_OK;
 }
 
@@ -1104,7 +1104,7 @@ int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& 
   static bool attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
-    a, b.positions, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
+    a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride);
   return LBT_OK;
 }

@@ -352,7 +352,7 @@ struct HistBatch {
   int F;
   const int2* qgh;
   int K;
-  const int2* positions;
+  const int32_t* rows;  // row numbers in node order (the level's segments index into it)
   const int32_t* seg;
   int j0;
   int n_nodes;
