@@ -1184,6 +1184,7 @@ struct Layout {
   int32_t* tile_start;
   int4* tiles;
   LevelMeta* meta;
+  int32_t* pair_sync;
   LevelMeta* level_totals;
   Cand* partial;
   I64Pair* hist;
@@ -1256,6 +1257,7 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   // a tile holds at least 8 rows (two rows per pass, four passes); every node adds at most one partial tile
   L.tiles         = ar.take<int4>(N / 8 + level_nodes + 1);
   L.meta          = ar.take<LevelMeta>(1);
+  L.pair_sync     = ar.take<int32_t>(kPairSyncSlots);
   L.level_totals  = ar.take<LevelMeta>(max_depth > 0 ? max_depth : 1);
   const int64_t max_chunks = (static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk;
   L.partial       = ar.take<Cand>(level_nodes * max_chunks);
@@ -1383,6 +1385,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.bins_t        = L.binned != nullptr ? L.bins_t : nullptr;
   hs.bins_t_stride = L.bins_t_stride;
   hs.meta       = L.meta;
+  hs.pair_sync  = L.pair_sync;
   LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
 
   const uint64_t max_bytes = prm.hist_cache_bytes > 0 ? static_cast<uint64_t>(prm.hist_cache_bytes) : 1000000000ULL;

@@ -46,6 +46,8 @@ constexpr int kSmallNodeRows = 64;  // below this a node goes straight to global
 constexpr int kUnroll        = 4;   // rows per lane and tile, search kernels
 constexpr int kBinnedUnroll  = 8;   // rows per lane and tile, histogram kernel (halved for 16-byte loads)
 constexpr int kLinearProbes  = 8;   // forward probes before falling back to a binary search
+constexpr int kPairSyncTiles = 8;   // tiles between two meeting points of the root launch's workgroups
+constexpr int kPairSyncSpins = 64;  // polls (about 0.9 us apart) a workgroup waits at one
 constexpr int kProbePad      = 3;   // +inf entries behind every feature's proposals in the binning pass
 constexpr int kProbeSlack    = 8;   // further entries behind the last feature that a probe window may touch
 
@@ -116,8 +118,11 @@ __global__ void __launch_bounds__(kPlanThreads)
 // (node, first row, end row, rows of the node), indexed like the tiles.
 __global__ void __launch_bounds__(kPlanThreads)
   expand_tiles_kernel(int j0, int n_nodes, int level_first, const int32_t* seg, const int32_t* tile_start,
-                      const LevelMeta* meta, int tile_rows, int4* tiles)
+                      const LevelMeta* meta, int tile_rows, int4* tiles, int32_t* pair_sync)
 {
+  // the arrival counters of the launch that follows start from zero
+  if (blockIdx.x == 0 && pair_sync != nullptr)
+    for (int i = threadIdx.x; i < kPairSyncSlots; i += kPlanThreads) pair_sync[i] = 0;
   const int tile = blockIdx.x * kPlanThreads + threadIdx.x;
   if (tile >= meta->n_tiles) return;
   // last j with tile_start[j] <= tile
@@ -863,7 +868,8 @@ __device__ __forceinline__ void turn_bytes(uint32_t w0, uint32_t w1, uint32_t w2
 template <typename BinT, int BV, bool kEmbed, bool kRoot>
 __global__ void __launch_bounds__(kHistThreads)
   binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
-                          const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride)
+                          const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride,
+                          int32_t* pair_sync)
 {
   using Word = typename BinVec<BinT, BV>::type;
   constexpr int kRows = kRoot ? 4 : (BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll);  // rows per lane and tile
@@ -954,6 +960,25 @@ __global__ void __launch_bounds__(kHistThreads)
   }
 
   for (int tile = t_begin; tile < t_end; tile++) {
+    if constexpr (kRoot) {
+      // The workgroups of the feature groups (and outputs) that walk the same rows read the
+      // same cache lines (a row's records share a line). Every kPairSyncTiles tiles each one
+      // counts itself in and gives the others a bounded time to catch up, so that the line one
+      // of them fetched is still in the L2 when the next one asks for it. Only a hint: after
+      // kPairSyncSpins polls a workgroup goes on regardless.
+      const int done = tile - t_begin;
+      if (pair_sync != nullptr && done > 0 && done % kPairSyncTiles == 0) {
+        if (threadIdx.x == 0) {
+          const int want = done / kPairSyncTiles * w.n_gk;
+          __hip_atomic_fetch_add(pair_sync + chunk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int spin = 0; spin < kPairSyncSpins; spin++) {
+            if (__hip_atomic_load(pair_sync + chunk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= want) break;
+            __builtin_amdgcn_s_sleep(32);
+          }
+        }
+        __syncthreads();
+      }
+    }
     if (tile + 1 < t_end) load_data(row_n, b_n, q_n);
     if (tile + 2 < t_end) {
       tnn      = win.get(tile + 2);
@@ -1105,7 +1130,8 @@ int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& 
   LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
-    static_cast<BinT*>(hs.bins_t), hs.bins_t_stride);
+    static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
+    kRoot && a.w.n_gk > 1 && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr);
   return LBT_OK;
 }
 template <typename BinT, int BV, bool kEmbed>
@@ -1201,7 +1227,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
     expand_tiles_kernel<<<static_cast<unsigned>((max_tiles + kPlanThreads - 1) / kPlanThreads), kPlanThreads, 0,
                           stream>>>(b.j0, b.n_nodes, b.level_first, b.seg, hs.tile_start, hs.meta, w.tile_rows,
-                                    hs.tiles);
+                                    hs.tiles, root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr);
   }
   ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   if (use_cache) {

@@ -307,6 +307,7 @@ struct HistSetup {
   int32_t* tile_start = nullptr;
   int4* tiles         = nullptr;  // one descriptor per tile of the batch in flight
   LevelMeta* meta    = nullptr;
+  int32_t* pair_sync = nullptr;  // kPairSyncSlots arrival counters of the root launch's row ranges
   // bin cache: written by the root binning pass and read by the histogram kernel of every
   // level instead of X; stored histogram group by histogram group as [group][row][record]
   void* binned         = nullptr;  // null: cache off
@@ -329,6 +330,7 @@ struct HistSetup {
 };
 
 constexpr int kMaxCells = 16384;  // table cells per feature at most (one 32-bit word per 16 cells)
+constexpr int kPairSyncSlots = 4096;
 constexpr int kHistThreads       = 1024;
 // LDS a histogram-stage workgroup may fill; 4 KB of the 160 KB stay free for the tile window
 constexpr size_t kLdsBudget = 160 * 1024 - 512 - 4096;
