@@ -483,20 +483,33 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
 {
   *ens = lbt_packed_ensemble{};
   if (buffer == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
-  size_t x_bytes  = 0;
-  const int lanes = tile_lanes<T>(F, &x_bytes);
-  if (lanes == 0) return LBT_OK;
-  const int batch_trees = lanes == 4 ? TileShape<4>::kBatchTrees
-                                     : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees);
-  constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
-  const int64_t node_cap = std::min<int64_t>(static_cast<int64_t>((kTileLds - x_bytes) / sizeof(PackedNode<T>)),
-                                             static_cast<int64_t>(kCopyWords) * kTileThreads * kNodesPerWord);
   int64_t total_nodes = 0;
   int max_nodes       = 0;
   for (int i = 0; i < n_trees; i++) {
     total_nodes += tree_nodes[i];
     max_nodes = std::max(max_nodes, tree_nodes[i]);
   }
+  size_t x_bytes = 0;
+  int lanes      = tile_lanes<T>(F, &x_bytes);
+  if (lanes == 0) return LBT_OK;
+  // A small ensemble spends its time streaming X: then a narrower row tile that lets two
+  // workgroups share a CU (one loads while the other walks) beats the widest tile that fits.
+  const size_t all_nodes = static_cast<size_t>(total_nodes + 2 * n_trees) * sizeof(PackedNode<T>);
+  if (all_nodes <= 24 * 1024) {
+    for (int l : {4, 8, 16}) {
+      const size_t xb = (static_cast<size_t>(kTileThreads / l) * (F | 1) * sizeof(T) + 15) & ~size_t(15);
+      if (l >= lanes && xb + all_nodes <= 78 * 1024) {
+        lanes   = l;
+        x_bytes = xb;
+        break;
+      }
+    }
+  }
+  const int batch_trees = lanes == 4 ? TileShape<4>::kBatchTrees
+                                     : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees);
+  constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
+  const int64_t node_cap = std::min<int64_t>(static_cast<int64_t>((kTileLds - x_bytes) / sizeof(PackedNode<T>)),
+                                             static_cast<int64_t>(kCopyWords) * kTileThreads * kNodesPerWord);
   if (max_nodes > node_cap || max_nodes > kMaxPackedNodes) return LBT_OK;
   const size_t need = packed_bytes(n_trees, total_nodes, K, sizeof(PackedNode<T>));
   if (buffer_bytes < need) {
@@ -509,7 +522,7 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
   std::vector<BatchInfo> binfo;
   std::vector<int64_t> node_off(n_trees);
   std::vector<int32_t> rel_off(n_trees);
-  int64_t off = 0;
+  int64_t off = 0, widest_batch = 0;
   for (int t = 0; t < n_trees;) {
     off = (off + kNodesPerWord - 1) / kNodesPerWord * kNodesPerWord;  // 16-byte aligned start
     BatchInfo bi{};
@@ -528,6 +541,7 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
     }
     bi.total = static_cast<int32_t>(in_batch);
     off += in_batch;
+    widest_batch = std::max(widest_batch, in_batch);
     binfo.push_back(bi);
   }
   for (int first = 0; first < n_trees; first += kPackTrees) {
@@ -562,6 +576,9 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
   ens->n_trees     = n_trees;
   ens->n_batches   = n_batches;
   ens->lanes       = lanes;
+  // the row tile and the widest batch of nodes (whole 16-byte words)
+  ens->lds_bytes   = static_cast<int32_t>(
+    x_bytes + ((static_cast<size_t>(widest_batch + kNodesPerWord) * sizeof(PackedNode<T>) + 15) & ~size_t(15)));
   ens->total_nodes = total_nodes;
   return LBT_OK;
 }
@@ -578,7 +595,7 @@ int run_tiled(hipStream_t stream, const T* X, int64_t N, const lbt_packed_ensemb
   const unsigned tiles = static_cast<unsigned>((N + tile_rows - 1) / tile_rows);
   auto launch = [&](auto kernel, bool (&flags)[kMaxDevices]) -> int {
     LBT_TRY(allow_dynamic_lds(kernel, kTileLds, flags));
-    kernel<<<tiles, kTileThreads, kTileLds, stream>>>(X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes,
+    kernel<<<tiles, kTileThreads, static_cast<size_t>(ens.lds_bytes), stream>>>(X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes,
                                                       lay.leaves, K, out);
     return LBT_OK;
   };
@@ -792,7 +809,8 @@ int lbt_predict_packed(void* stream, const void* X, int32_t x_dtype, int64_t n_r
   LBT_REQUIRE((ensemble->lanes == 4 || ensemble->lanes == 8 || ensemble->lanes == 16) && ensemble->n_trees >= 1 &&
                 ensemble->n_batches >= 1 && ensemble->n_batches <= ensemble->n_trees &&
                 ensemble->n_outputs >= 1 && ensemble->n_outputs <= lbt::kTileMaxK &&
-                ensemble->total_nodes >= ensemble->n_trees,
+                ensemble->total_nodes >= ensemble->n_trees && ensemble->lds_bytes >= 16 &&
+                static_cast<size_t>(ensemble->lds_bytes) <= lbt::kTileLds,
               "corrupt ensemble descriptor");
   LBT_REQUIRE(ensemble->bytes >= lbt_predict_workspace_bytes(ensemble->n_trees, ensemble->total_nodes,
                                                              ensemble->n_outputs, ensemble->x_dtype),

@@ -78,6 +78,8 @@ class PackedEnsemble(C.Structure):
         ("n_trees", C.c_int32),
         ("n_batches", C.c_int32),
         ("lanes", C.c_int32),
+        ("lds_bytes", C.c_int32),
+        ("reserved", C.c_int32),
         ("total_nodes", C.c_int64),
     ]
 
