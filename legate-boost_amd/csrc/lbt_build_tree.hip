@@ -125,7 +125,7 @@ __global__ void __launch_bounds__(kThreads)
   sort_unique_kernel(const T* draft, int S, int P, T* uniq, int32_t* counts)
 {
   using Key = typename KeyOf<T>::type;
-  extern __shared__ unsigned char smem_raw[];
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   Key* keys       = reinterpret_cast<Key*>(smem_raw);
   __shared__ int s_cnt[kThreads];
   const int f     = blockIdx.x;
@@ -1185,6 +1185,10 @@ struct Layout {
   int4* tiles;
   LevelMeta* meta;
   int32_t* pair_sync;
+  unsigned long long* partials;
+  int32_t* partial_lists;
+  int32_t* partial_list_count;
+  int32_t* partial_count;
   LevelMeta* level_totals;
   Cand* partial;
   I64Pair* hist;
@@ -1258,6 +1262,12 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.tiles         = ar.take<int4>(N / 8 + level_nodes + 1);
   L.meta          = ar.take<LevelMeta>(1);
   L.pair_sync     = ar.take<int32_t>(kPairSyncSlots);
+  // parked sub-histograms of a launch on cached bins (kPartialSlots of the widest group the LDS can hold)
+  L.partials      = max_depth >= 2 ? ar.take<unsigned long long>(static_cast<size_t>(kPartialSlots) * kPartialStrideMax)
+                                   : nullptr;
+  L.partial_lists = ar.take<int32_t>(static_cast<size_t>(kPartialMaxLists) * kPartialListCap);
+  L.partial_list_count = ar.take<int32_t>(kPartialMaxLists);
+  L.partial_count = ar.take<int32_t>(1);
   L.level_totals  = ar.take<LevelMeta>(max_depth > 0 ? max_depth : 1);
   const int64_t max_chunks = (static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk;
   L.partial       = ar.take<Cand>(level_nodes * max_chunks);
@@ -1386,6 +1396,11 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.bins_t_stride = L.bins_t_stride;
   hs.meta       = L.meta;
   hs.pair_sync  = L.pair_sync;
+  hs.partials      = L.partials;
+  hs.partial_lists = L.partial_lists;
+  hs.partial_list_count = L.partial_list_count;
+  hs.partial_count = L.partial_count;
+  hs.partial_slots = kPartialSlots;
   LBT_TRY(hist_prepare(stream, hs, sizeof(T) == 8, F, K, N, rp, L.proposals, L.row_pointers, X));
 
   const uint64_t max_bytes = prm.hist_cache_bytes > 0 ? static_cast<uint64_t>(prm.hist_cache_bytes) : 1000000000ULL;

@@ -118,11 +118,16 @@ __global__ void __launch_bounds__(kPlanThreads)
 // (node, first row, end row, rows of the node), indexed like the tiles.
 __global__ void __launch_bounds__(kPlanThreads)
   expand_tiles_kernel(int j0, int n_nodes, int level_first, const int32_t* seg, const int32_t* tile_start,
-                      const LevelMeta* meta, int tile_rows, int4* tiles, int32_t* pair_sync)
+                      const LevelMeta* meta, int tile_rows, int4* tiles, int32_t* pair_sync, int32_t* partial_count,
+                      int32_t* partial_list_count)
 {
   // the arrival counters of the launch that follows start from zero
   if (blockIdx.x == 0 && pair_sync != nullptr)
     for (int i = threadIdx.x; i < kPairSyncSlots; i += kPlanThreads) pair_sync[i] = 0;
+  if (blockIdx.x == 0 && partial_count != nullptr) {
+    if (threadIdx.x == 0) *partial_count = 0;
+    for (int i = threadIdx.x; i < kPartialMaxLists; i += kPlanThreads) partial_list_count[i] = 0;
+  }
   const int tile = blockIdx.x * kPlanThreads + threadIdx.x;
   if (tile >= meta->n_tiles) return;
   // last j with tile_start[j] <= tile
@@ -349,7 +354,11 @@ __device__ inline int count_less(const T* p, int n, T x, int steps)
 // Merge of the packed LDS sub-histogram into the int64 histogram of a node.
 __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst)
 {
-  for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+  // Workgroups that finish a node together would walk its bins in step and queue up on the
+  // same cache lines: each one starts at a place of its own and wraps around.
+  const int start = static_cast<int>((blockIdx.x * 2654435761u) % static_cast<unsigned>(nb));
+  for (int t = threadIdx.x; t < nb; t += kHistThreads) {
+    const int i          = t + start < nb ? t + start : t + start - nb;
     unsigned long long v = s_hist[i];
     if (v != 0) {
       int32_t gv  = static_cast<int32_t>(v >> 32);
@@ -361,12 +370,123 @@ __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I
   }
 }
 
+// Where the workgroups of a launch park their sub-histograms for reduce_partials_kernel.
+struct PartialSink {
+  unsigned long long* partials;
+  int32_t* lists;       // [list][kPartialListCap] slots of the list (node of the batch, group, output)
+  int32_t* list_count;  // [list]
+  int32_t* count;       // slots handed out
+  int slots;            // 0: merge with atomics
+  int stride;           // packed bins per slot
+};
+
+// Hands the packed sub-histogram over instead of adding it bin by bin: two 64-bit global
+// atomics per bin and workgroup were a quarter of the histogram stage (the L2 completes about
+// 5e10 of them per second). A workgroup takes a slot, copies its bins there as they are and
+// clears them; a pass after the launch adds up the slots of every (node, group, output) with
+// plain loads. Without a free slot the atomics do it. All threads of the workgroup call this.
+__device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst, const PartialSink& sink,
+                                          int tag, int* s_slot, bool sole_owner)
+{
+  if (sole_owner) {
+    // every row of the node went through this workgroup: nobody else adds to these bins
+    for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+      const unsigned long long v = s_hist[i];
+      if (v != 0) {
+        I64Pair p = dst[i];
+        p.grad += static_cast<int32_t>(v >> 32);
+        p.hess += static_cast<uint32_t>(v);
+        dst[i]    = p;
+        s_hist[i] = 0;
+      }
+    }
+    return;
+  }
+  int slot = sink.slots;
+  if (sink.slots > 0) {
+    if (threadIdx.x == 0) {
+      // a slot, and a place for it in the list of its (node, group, output)
+      int got = atomicAdd(sink.count, 1);
+      if (got < sink.slots) {
+        const int at = atomicAdd(sink.list_count + tag, 1);
+        if (at < kPartialListCap)
+          sink.lists[static_cast<int64_t>(tag) * kPartialListCap + at] = got;
+        else
+          got = sink.slots;  // list full: this one goes the slow way
+      }
+      *s_slot = got;
+    }
+    __syncthreads();
+    slot = *s_slot;
+  }
+  if (slot < sink.slots) {
+    unsigned long long* out = sink.partials + static_cast<int64_t>(slot) * sink.stride;
+    for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+      out[i]    = s_hist[i];
+      s_hist[i] = 0;
+    }
+  } else {
+    merge_sub_histogram(s_hist, nb, dst);
+  }
+}
+
+// Adds up the parked sub-histograms. Workgroup (x, y, z): bins x * 1024 .. of the list y =
+// (node of the batch, group, output), every gridDim.z-th slot of the list starting with the
+// z-th. With one workgroup per bin range (gridDim.z == 1) the totals are added plainly, no
+// other workgroup touches those bins; a long list split over several workgroups (few lists:
+// the levels near the root) adds them with atomics. Integer sums: any order gives the same.
+__global__ void __launch_bounds__(kHistThreads)
+  reduce_partials_kernel(PartialSink sink, int K, int n_groups, const int32_t* __restrict__ groups,
+                         const int32_t* __restrict__ row_pointers, HistView hist, int first_node)
+{
+  const int tag = blockIdx.y;
+  const int m   = min(sink.list_count[tag], kPartialListCap);
+  if (static_cast<int>(blockIdx.z) >= m) return;
+  const int n_gk  = n_groups * K;
+  const int node  = first_node + tag / n_gk;
+  const int gk    = tag - tag / n_gk * n_gk;
+  const int group = gk / K, k = gk - gk / K * K;
+  const int bin0  = row_pointers[groups[group]];
+  const int nb    = row_pointers[groups[group + 1]] - bin0;
+  const int bin   = blockIdx.x * kHistThreads + threadIdx.x;
+  if (bin >= nb) return;
+  const int32_t* __restrict__ list = sink.lists + static_cast<int64_t>(tag) * kPartialListCap;
+  const unsigned long long* src    = sink.partials + bin;
+  const int step                   = gridDim.z;
+  int64_t g = 0, h = 0;
+  int i = blockIdx.z;
+  // eight slots at a time, so that their loads are in flight together
+  for (; i + 7 * step < m; i += 8 * step) {
+    unsigned long long v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) v[u] = src[static_cast<int64_t>(list[i + u * step]) * sink.stride];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      g += static_cast<int32_t>(v[u] >> 32);
+      h += static_cast<uint32_t>(v[u]);
+    }
+  }
+  for (; i < m; i += step) {
+    const unsigned long long v = src[static_cast<int64_t>(list[i]) * sink.stride];
+    g += static_cast<int32_t>(v >> 32);
+    h += static_cast<uint32_t>(v);
+  }
+  I64Pair* dst = hist.at(node, k, bin0 + bin);
+  if (step == 1) {
+    dst->grad += g;
+    dst->hess += h;
+  } else {
+    if (g != 0) atomic_add_i64(&dst->grad, g);
+    if (h != 0) atomic_add_i64(&dst->hess, h);
+  }
+}
+
 template <typename T, int VEC, bool kIdentityRows>
 __global__ void __launch_bounds__(kHistThreads)
   histogram_kernel(HistArgs<T> a, LBT_WALK_PARAMS, const T* __restrict__ X, const int2* __restrict__ qgh)
 {
   using Vec = typename VecOf<T, VEC>::type;
-  extern __shared__ unsigned char smem_raw[];
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   const TileWalk& w = a.w;
 
   // workgroup -> (row-tile range, group, output). Linear workgroup ids are dealt
@@ -603,7 +723,7 @@ __global__ void __launch_bounds__(kHistThreads)
                   BinT* __restrict__ binned)
 {
   using Vec = typename VecOf<T, VEC>::type;
-  extern __shared__ unsigned char smem_raw[];
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   const int xcd   = blockIdx.x & 7;
   const int slot  = blockIdx.x >> 3;
   const int group = slot % a.n_sgroups;
@@ -869,11 +989,12 @@ template <typename BinT, int BV, bool kEmbed, bool kRoot>
 __global__ void __launch_bounds__(kHistThreads)
   binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
                           const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride,
-                          int32_t* pair_sync)
+                          int32_t* pair_sync, PartialSink sink)
 {
+  __shared__ int s_slot;
   using Word = typename BinVec<BinT, BV>::type;
   constexpr int kRows = kRoot ? 4 : (BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll);  // rows per lane and tile
-  extern __shared__ unsigned char smem_raw[];
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   const TileWalk& w = a.w;
   const int xcd   = blockIdx.x & 7;
   const int slot  = blockIdx.x >> 3;
@@ -910,6 +1031,11 @@ __global__ void __launch_bounds__(kHistThreads)
   const int t_end   = static_cast<int>(static_cast<int64_t>(n_tiles) * (chunk + 1) / w.n_chunks);
   int cur_node           = -1;
   unsigned long long acc = 0;
+  // rows of cur_node that this workgroup has taken, and how many the node has: when they
+  // agree at the end of the node, its bins belong to this workgroup alone. Not when single
+  // tiles may go to the histogram directly (huge gradients), which other workgroups may do too.
+  int node_rows = 0, node_total = 0;
+  const bool owners = static_cast<unsigned long long>(w.tile_rows) * max_abs <= 2147483647ULL;
   __syncthreads();
 
   auto load_rows = [&](const Tile& t, int (&row)[kRows]) -> unsigned {
@@ -990,12 +1116,20 @@ __global__ void __launch_bounds__(kHistThreads)
     if (!direct) {
       if (tc.node != cur_node || (acc + nrows) * max_abs > 2147483647ULL) {
         __syncthreads();
-        if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
+        if (cur_node >= 0)
+          park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink,
+                             (cur_node - w.level_first - w.j0) * w.n_gk + gk, &s_slot,
+                             owners && tc.node != cur_node && node_rows == node_total);
         __syncthreads();
+        if (tc.node != cur_node) {
+          node_rows  = 0;
+          node_total = tc.seg_rows;
+        }
         cur_node = tc.node;
         acc      = 0;
       }
       acc += nrows;
+      node_rows += nrows;
     }
     if constexpr (kEmbed && BV == 16) {
 #pragma unroll
@@ -1085,7 +1219,9 @@ __global__ void __launch_bounds__(kHistThreads)
     }
   }
   __syncthreads();
-  if (cur_node >= 0) merge_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0));
+  if (cur_node >= 0)
+    park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink, (cur_node - w.level_first - w.j0) * w.n_gk + gk,
+                       &s_slot, owners && node_rows == node_total);
 }
 
 template <typename T, int VEC, bool kIdentityRows>
@@ -1126,12 +1262,25 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
 template <typename BinT, int BV, bool kEmbed, bool kRoot>
 int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
 {
+  PartialSink sink{hs.partials, hs.partial_lists, hs.partial_list_count, hs.partial_count, 0, hs.partial_stride};
+  if (hs.partials != nullptr && static_cast<int64_t>(a.w.n_nodes) * a.w.n_gk <= kPartialMaxLists)
+    sink.slots = hs.partial_slots;
   static bool attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
-    kRoot && a.w.n_gk > 1 && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr);
+    kRoot && a.w.n_gk > 1 && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr, sink);
+  if (sink.slots > 0) {
+    // the stride is the widest group in bins; near the root, where few lists are long, the slots of
+    // a list are dealt to several workgroups
+    const int lists      = a.w.n_nodes * a.w.n_gk;
+    const int bin_chunks = (sink.stride + kHistThreads - 1) / kHistThreads;
+    const int split      = std::max(1, std::min(16, 256 / (lists * bin_chunks)));
+    dim3 rgrid(static_cast<unsigned>(bin_chunks), static_cast<unsigned>(lists), static_cast<unsigned>(split));
+    reduce_partials_kernel<<<rgrid, kHistThreads, 0, stream>>>(sink, a.K, a.w.n_gk / a.K, a.groups, a.row_pointers,
+                                                               a.hist, a.w.level_first + a.w.j0);
+  }
   return LBT_OK;
 }
 template <typename BinT, int BV, bool kEmbed>
@@ -1227,7 +1376,8 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
     expand_tiles_kernel<<<static_cast<unsigned>((max_tiles + kPlanThreads - 1) / kPlanThreads), kPlanThreads, 0,
                           stream>>>(b.j0, b.n_nodes, b.level_first, b.seg, hs.tile_start, hs.meta, w.tile_rows,
-                                    hs.tiles, root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr);
+                                    hs.tiles, root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr,
+                                    use_cache ? hs.partial_count : nullptr, hs.partial_list_count);
   }
   ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   if (use_cache) {
@@ -1409,6 +1559,8 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     }
     hs.n_groups   = static_cast<int>(groups.size()) - 1;
     hs.blds_bytes = (blds + 8 * kHistThreads + 15) & ~size_t(15);
+    hs.partial_stride = static_cast<int>(blds / 8);  // bins of the widest group
+    if (hs.partial_stride > kPartialStrideMax) hs.partials = nullptr;
     hs.brpp       = rows_per_pass(groups, hs.bvec);
     LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
     // record layout of every histogram group

@@ -308,6 +308,15 @@ struct HistSetup {
   int4* tiles         = nullptr;  // one descriptor per tile of the batch in flight
   LevelMeta* meta    = nullptr;
   int32_t* pair_sync = nullptr;  // kPairSyncSlots arrival counters of the root launch's row ranges
+  // sub-histograms parked for the reduction pass: slot s holds partial_stride packed bins
+  unsigned long long* partials = nullptr;
+  // the slots of list t = (node of the batch) * groups * outputs + group * outputs + output:
+  // partial_lists[t * kPartialListCap ..], partial_list_count[t] of them
+  int32_t* partial_lists = nullptr;
+  int32_t* partial_list_count = nullptr;  // [kPartialMaxLists]
+  int32_t* partial_count = nullptr;  // slots handed out by the running launch
+  int partial_slots = 0;
+  int partial_stride = 0;
   // bin cache: written by the root binning pass and read by the histogram kernel of every
   // level instead of X; stored histogram group by histogram group as [group][row][record]
   void* binned         = nullptr;  // null: cache off
@@ -331,6 +340,11 @@ struct HistSetup {
 
 constexpr int kMaxCells = 16384;  // table cells per feature at most (one 32-bit word per 16 cells)
 constexpr int kPairSyncSlots = 4096;
+// bins of the widest feature group that fits the LDS beside the lanes' spare slots
+constexpr int kPartialStrideMax = (160 * 1024 - 512 - 4096 - 8 * 1024) / 8;
+constexpr int kPartialSlots = 1024;      // sub-histograms one launch can park
+constexpr int kPartialListCap = 320;      // slots one list can index (a node's row ranges plus overflow merges)
+constexpr int kPartialMaxLists = 4096;   // (node, group, output) triples the reduction pass is launched for
 constexpr int kHistThreads       = 1024;
 // LDS a histogram-stage workgroup may fill; 4 KB of the 160 KB stay free for the tile window
 constexpr size_t kLdsBudget = 160 * 1024 - 512 - 4096;

@@ -321,7 +321,7 @@ __global__ void __launch_bounds__(kTileThreads)
 {
   using S = TileShape<L>;
   constexpr int kTileRows = S::kRows, kLaneTrees = S::kLaneTrees;
-  extern __shared__ unsigned char smem_raw[];
+  extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   T* s_x = reinterpret_cast<T*>(smem_raw);
   const size_t x_bytes = (static_cast<size_t>(kTileRows) * pitch * sizeof(T) + 15) & ~size_t(15);
   PackedNode<T>* s_nodes = reinterpret_cast<PackedNode<T>*>(smem_raw + x_bytes);
