@@ -164,7 +164,7 @@ def bench_training(args):
             # build: same values as PredictTask on the training rows (checked bit for bit in the tests)
             g, h = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc, pred,
                                          None, lr, out=gh)
-            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True)
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True, wait=False)
             ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         return r
 

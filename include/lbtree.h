@@ -108,6 +108,23 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
                    double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
                    void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
 
+/*
+ * lbt_build_tree without the wait at the end: the call returns once the last kernel is
+ * enqueued (it still waits once, early on, for the bin counts of the split proposals, which
+ * decide the kernels' layout). Outputs, workspace and device taps are valid in stream order,
+ * which is all a consumer on the same stream (PredictTask, lbt_add_leaf_values, the next
+ * lbt_build_tree on the same workspace) needs; the reference synchronises (build_tree.cu:1356)
+ * although Legate orders tasks on the task stream. The members of `taps` that hold host
+ * values read back from the device (scales, level_instances, level_built_instances,
+ * level_built_nodes) are not filled. Errors of kernels surface at the caller's next
+ * synchronisation.
+ */
+int lbt_build_tree_async(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
+                         int64_t n_rows, int32_t n_features, const double* g, const double* h,
+                         int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
+                         double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
+                         void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
+
 /* Device scratch for lbt_predict: room for the ensemble packed into one node array and one
  * leaf array (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
 size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype);
@@ -272,7 +289,9 @@ typedef struct lbt_profile {
 
 /* on = 1: lbt_build_tree / lbt_predict bracket every kernel class with HIP events on the
  * stream of the call (about 0.3 ms of a 6 ms build); on = 2: only the two histogram-stage
- * classes (LBT_PROF_BINNING, LBT_PROF_HISTOGRAM); 0: off. Counters accumulate until reset. */
+ * classes (LBT_PROF_BINNING, LBT_PROF_HISTOGRAM); 0: off. Counters accumulate until reset.
+ * lbt_profile_get and lbt_profile_reset wait for the events of calls that returned without
+ * synchronising (lbt_build_tree_async, lbt_predict). */
 void lbt_profile_enable(int on);
 void lbt_profile_reset(void);
 void lbt_profile_get(lbt_profile* out);

@@ -1293,11 +1293,37 @@ int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
 }
 
 
+// What the host reads back in the middle of a call (bin counts per feature, the quantiser's
+// overflow flag): pinned memory and two events per host thread, so that each value is waited
+// for by itself and not together with everything else that is queued on the stream.
+struct HostMirror {
+  int32_t* pinned = nullptr;  // [4 + capacity]: two 64-bit quantiser statistics, then the row pointers
+  size_t capacity = 0;
+  hipEvent_t counts_here = nullptr, stats_here = nullptr;
+};
+
+int host_mirror(int F, HostMirror** out)
+{
+  static thread_local HostMirror hm;
+  if (hm.counts_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.counts_here, hipEventDisableTiming));
+  if (hm.stats_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.stats_here, hipEventDisableTiming));
+  const size_t need = static_cast<size_t>(F) + 1;
+  if (hm.capacity < need) {
+    if (hm.pinned != nullptr) LBT_HIP(hipHostFree(hm.pinned));
+    hm.pinned   = nullptr;
+    hm.capacity = 0;
+    LBT_HIP(hipHostMalloc(reinterpret_cast<void**>(&hm.pinned), sizeof(int32_t) * (4 + need), hipHostMallocDefault));
+    hm.capacity = need;
+  }
+  *out = &hm;
+  return LBT_OK;
+}
+
 template <typename T>
 int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F,
                     const double* g, const double* h, int K, const uint8_t* feature_set,
                     const lbt_build_params& prm, double* leaf, int32_t* feature, double* split,
-                    double* gain, double* hessian, Layout& L, lbt_build_taps* taps)
+                    double* gain, double* hessian, Layout& L, lbt_build_taps* taps, bool sync_at_end)
 {
   const int max_depth = prm.max_depth;
   const int max_nodes = prm.max_nodes;
@@ -1311,7 +1337,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   }
 
   // ---- split proposals
-  std::vector<int32_t> rp(F + 1);
+  HostMirror* hm = nullptr;
+  LBT_TRY(host_mirror(F, &hm));
+  int32_t* const rp_here = hm->pinned + 4;
   {
     ProfScope ps(LBT_PROF_PROPOSALS, stream);
     T* draft = static_cast<T*>(L.draft);
@@ -1326,7 +1354,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     row_pointers_kernel<<<1, 64, 0, stream>>>(L.counts, F, L.row_pointers);
     compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(
       uniq, S, L.row_pointers, static_cast<T*>(L.proposals), L.bin_feature);
-    LBT_HIP(hipMemcpyAsync(rp.data(), L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
+    LBT_HIP(hipMemcpyAsync(rp_here, L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
+    LBT_HIP(hipEventRecord(hm->counts_here, stream));
   }
   // ---- quantiser
   {
@@ -1356,8 +1385,22 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization);
   }
-  unsigned long long h_qstats[2] = {0, 0};
-  LBT_HIP(hipMemcpyAsync(h_qstats, L.qstats, sizeof(h_qstats), hipMemcpyDeviceToHost, stream));
+  const unsigned long long* const h_qstats = reinterpret_cast<const unsigned long long*>(hm->pinned);
+  LBT_HIP(hipMemcpyAsync(hm->pinned, L.qstats, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, stream));
+  LBT_HIP(hipEventRecord(hm->stats_here, stream));
+  bool stats_checked = false;
+  // a gradient that does not fit 32 bits ends the call; asked once a level's work is queued,
+  // when the answer has long arrived
+  auto check_stats = [&]() -> int {
+    if (stats_checked) return LBT_OK;
+    stats_checked = true;
+    LBT_HIP(hipEventSynchronize(hm->stats_here));
+    if (h_qstats[1] != 0) {
+      set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
+      return LBT_ERR_UNSUPPORTED;
+    }
+    return LBT_OK;
+  };
 
   // ---- positions and histogram cache (TreeBuilder ctor, build_tree.cu:997-1017)
   fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.rows[0], N, L.seg[0], L.block_seg[0],
@@ -1365,14 +1408,11 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
   if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
 
-  // the one host wait before the levels: the bin counts decide the feature groups, and a
-  // gradient that does not fit 32 bits ends the call. The quantiser above keeps the GPU busy
-  // while the host waits.
-  LBT_HIP(hipStreamSynchronize(stream));
-  if (h_qstats[1] != 0) {
-    set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
-    return LBT_ERR_UNSUPPORTED;
-  }
+  // the one host wait before the levels: the bin counts decide the feature groups. Only the
+  // copy of the counts is waited for; the quantiser queued behind it keeps the GPU busy while
+  // the host plans and queues the levels.
+  LBT_HIP(hipEventSynchronize(hm->counts_here));
+  const std::vector<int32_t> rp(rp_here, rp_here + F + 1);
   const int B = rp[F];
   proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
     static_cast<const T*>(L.proposals), B, L.proposals_d);
@@ -1511,7 +1551,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       cur_pos ^= 1;
       cur_seg ^= 1;
     }
+    if (depth == 0) LBT_TRY(check_stats());
   }
+  LBT_TRY(check_stats());
 
   if (row_leaf != nullptr) {
     ProfScope ps(LBT_PROF_POSITIONS, stream);
@@ -1548,15 +1590,33 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   }
 
   // ---- observation points
+  static_assert(sizeof(LevelMeta) == sizeof(LevelCounts), "the host mirror of LevelMeta");
+  const bool tap_levels =
+    taps && (taps->level_instances || taps->level_built_instances || taps->level_built_nodes) && max_depth > 0;
+  ProfLevels* prof_levels = nullptr;
+  if (profiler().mode != 0 && max_depth > 0) {
+    // bytes of one feature value as the level reads it (X itself, or its cached bin)
+    const bool cached      = hs.binned != nullptr;
+    const double per_value = cached ? hs.bin_bytes : static_cast<double>(sizeof(T));
+    prof_levels            = profiler().begin_levels(
+      std::min(max_depth, 64), static_cast<double>(F) * per_value + K * 8.0 + 8.0, static_cast<double>(K) * B * 16.0,
+      // the root launch also writes the feature-major copy of the bins
+      hs.bins_t != nullptr ? static_cast<double>(N) * F * hs.bin_bytes : 0.0);
+    if (prof_levels != nullptr) {
+      LBT_HIP(hipMemcpyAsync(prof_levels->host, L.level_totals, sizeof(LevelMeta) * prof_levels->levels,
+                             hipMemcpyDeviceToHost, stream));
+      LBT_HIP(hipEventRecord(prof_levels->arrived, stream));
+    }
+  }
   std::vector<LevelMeta> h_levels(max_depth > 0 ? max_depth : 1);
-  const bool want_levels = max_depth > 0 && ((profiler().mode != 0) || (taps && (taps->level_instances || taps->level_built_instances || taps->level_built_nodes)));
-  if (want_levels)
+  if (tap_levels && sync_at_end)
     LBT_HIP(hipMemcpyAsync(h_levels.data(), L.level_totals, sizeof(LevelMeta) * max_depth, hipMemcpyDeviceToHost, stream));
   if (taps) {
     taps->n_bins          = B;
     taps->hist_node_begin = hv.node_begin;
     taps->hist_node_end   = static_cast<int32_t>(std::max<int64_t>(hv.node_begin, std::min<int64_t>(hv.node_end, used_end)));
-    LBT_HIP(hipMemcpyAsync(taps->scales, L.scales, sizeof(double) * 4, hipMemcpyDeviceToHost, stream));
+    // host members that come from the device are filled only by the call that waits for them
+    if (sync_at_end) LBT_HIP(hipMemcpyAsync(taps->scales, L.scales, sizeof(double) * 4, hipMemcpyDeviceToHost, stream));
     if (taps->proposals)
       LBT_HIP(hipMemcpyAsync(taps->proposals, L.proposals, sizeof(T) * B, hipMemcpyDeviceToDevice, stream));
     if (taps->row_pointers)
@@ -1578,36 +1638,18 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
         LBT_HIP(hipMemcpyAsync(taps->histogram, L.hist, sizeof(int64_t) * need, hipMemcpyDeviceToDevice, stream));
     }
   }
+  LBT_HIP(hipGetLastError());
+  if (!sync_at_end) return LBT_OK;
   LBT_HIP(hipStreamSynchronize(stream));
   LBT_HIP(hipGetLastError());
-  if (want_levels) {
+  if (tap_levels) {
     for (int d = 0; d < max_depth; d++) {
-      if (taps && taps->level_instances) taps->level_instances[d] = h_levels[d].instances;
-      if (taps && taps->level_built_instances) taps->level_built_instances[d] = h_levels[d].built_instances;
-      if (taps && taps->level_built_nodes) taps->level_built_nodes[d] = static_cast<int32_t>(h_levels[d].built_nodes);
+      if (taps->level_instances) taps->level_instances[d] = h_levels[d].instances;
+      if (taps->level_built_instances) taps->level_built_instances[d] = h_levels[d].built_instances;
+      if (taps->level_built_nodes) taps->level_built_nodes[d] = static_cast<int32_t>(h_levels[d].built_nodes);
     }
   }
-  if ((profiler().mode != 0)) {
-    profiler().collect();
-    // algorithmic bytes of the histogram launches of each level:
-    // X rows of built nodes + their packed gradients + one position pair per
-    // instance + the built histograms written once
-    auto& acc = profiler().acc;
-    const bool cached = hs.binned != nullptr;
-    for (int d = 0; d < max_depth && d < 64; d++) {
-      // bytes of one feature value as the level reads it (X itself, or its cached bin)
-      double per_value = cached ? hs.bin_bytes : static_cast<double>(sizeof(T));
-      double by = static_cast<double>(h_levels[d].built_instances) * (static_cast<double>(F) * per_value + K * 8.0 + 8.0) +
-                  static_cast<double>(h_levels[d].built_nodes) * K * B * 16.0;
-      // the root launch also writes the feature-major copy of the bins
-      if (d == 0 && hs.bins_t != nullptr) by += static_cast<double>(N) * F * hs.bin_bytes;
-      acc.level_bytes[d] += by;
-      acc.level_instances[d] += static_cast<double>(h_levels[d].instances);
-      acc.level_built_instances[d] += static_cast<double>(h_levels[d].built_instances);
-      acc.level_built_nodes[d] += static_cast<double>(h_levels[d].built_nodes);
-      acc.bytes[LBT_PROF_HISTOGRAM] += by;
-    }
-  }
+  if (profiler().mode != 0) profiler().collect();
   return LBT_OK;
 }
 
@@ -1635,11 +1677,11 @@ size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_
   return ar.used + 256;
 }
 
-int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
-                   int64_t n_rows, int32_t n_features, const double* g, const double* h,
-                   int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
-                   double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
-                   void* workspace, size_t workspace_bytes, lbt_build_taps* taps)
+static int build_tree_entry(void* stream, const void* X, int32_t x_dtype, int64_t row_offset, int64_t n_rows,
+                            int32_t n_features, const double* g, const double* h, int32_t n_outputs,
+                            const uint8_t* feature_set, const lbt_build_params* params, double* leaf, int32_t* feature,
+                            double* split, double* gain, double* hessian, void* workspace, size_t workspace_bytes,
+                            lbt_build_taps* taps, bool sync_at_end)
 {
   LBT_TRY(lbt::validate(n_rows, n_features, n_outputs, params, x_dtype));
   LBT_REQUIRE(X && g && h && leaf && feature && split && gain && hessian, "null input or output pointer");
@@ -1663,16 +1705,36 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
   hipStream_t s = static_cast<hipStream_t>(stream);
   int rc;
   if (x_dtype == LBT_F32)
-    rc = lbt::build_tree_impl<float>(s, static_cast<const float*>(X), row_offset, n_rows, n_features, g, h,
-                                     n_outputs, feature_set, *params, leaf, feature, split, gain, hessian, L, taps);
+    rc = lbt::build_tree_impl<float>(s, static_cast<const float*>(X), row_offset, n_rows, n_features, g, h, n_outputs,
+                                     feature_set, *params, leaf, feature, split, gain, hessian, L, taps, sync_at_end);
   else
-    rc = lbt::build_tree_impl<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, g, h,
-                                      n_outputs, feature_set, *params, leaf, feature, split, gain, hessian, L, taps);
+    rc = lbt::build_tree_impl<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, g, h, n_outputs,
+                                      feature_set, *params, leaf, feature, split, gain, hessian, L, taps, sync_at_end);
   if (rc != LBT_OK && lbt::profiler().mode != 0) {
     (void)hipStreamSynchronize(s);
     lbt::profiler().collect();
   }
   return rc;
+}
+
+int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
+                   int64_t n_rows, int32_t n_features, const double* g, const double* h,
+                   int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
+                   double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
+                   void* workspace, size_t workspace_bytes, lbt_build_taps* taps)
+{
+  return build_tree_entry(stream, X, x_dtype, row_offset, n_rows, n_features, g, h, n_outputs, feature_set, params, leaf,
+                          feature, split, gain, hessian, workspace, workspace_bytes, taps, true);
+}
+
+int lbt_build_tree_async(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
+                         int64_t n_rows, int32_t n_features, const double* g, const double* h,
+                         int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,
+                         double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
+                         void* workspace, size_t workspace_bytes, lbt_build_taps* taps)
+{
+  return build_tree_entry(stream, X, x_dtype, row_offset, n_rows, n_features, g, h, n_outputs, feature_set, params, leaf,
+                          feature, split, gain, hessian, workspace, workspace_bytes, taps, false);
 }
 
 }  // extern "C"

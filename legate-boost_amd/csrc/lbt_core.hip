@@ -70,6 +70,50 @@ void Profiler::collect()
     pool.push_back(sp.stop);
   }
   open.clear();
+  for (auto& lv : levels) {
+    if (hipEventSynchronize(lv.arrived) == hipSuccess) {
+      for (int d = 0; d < lv.levels && d < 64; d++) {
+        const LevelCounts& c = lv.host[d];
+        // algorithmic bytes of the histogram launches of the level: the feature values and packed
+        // gradients of the rows of built nodes, one position per row, the built histograms once
+        double by = static_cast<double>(c.built_instances) * lv.bytes_per_built_row +
+                    static_cast<double>(c.built_nodes) * lv.bytes_per_built_node + (d == 0 ? lv.root_extra_bytes : 0.0);
+        acc.level_bytes[d] += by;
+        acc.level_instances[d] += static_cast<double>(c.instances);
+        acc.level_built_instances[d] += static_cast<double>(c.built_instances);
+        acc.level_built_nodes[d] += static_cast<double>(c.built_nodes);
+        acc.bytes[LBT_PROF_HISTOGRAM] += by;
+      }
+    }
+    pool.push_back(lv.arrived);
+    level_pool.push_back(lv.host);
+  }
+  levels.clear();
+}
+
+ProfLevels* Profiler::begin_levels(int n_levels, double per_row, double per_node, double root_extra)
+{
+  ProfLevels lv{};
+  if (!level_pool.empty()) {
+    lv.host = level_pool.back();
+    level_pool.pop_back();
+  } else if (hipHostMalloc(reinterpret_cast<void**>(&lv.host), sizeof(LevelCounts) * 64, hipHostMallocDefault) !=
+             hipSuccess) {
+    return nullptr;
+  }
+  if (!pool.empty()) {
+    lv.arrived = pool.back();
+    pool.pop_back();
+  } else if (hipEventCreate(&lv.arrived) != hipSuccess) {
+    level_pool.push_back(lv.host);
+    return nullptr;
+  }
+  lv.levels               = n_levels;
+  lv.bytes_per_built_row  = per_row;
+  lv.bytes_per_built_node = per_node;
+  lv.root_extra_bytes     = root_extra;
+  levels.push_back(lv);
+  return &levels.back();
 }
 
 }  // namespace lbt
@@ -85,11 +129,14 @@ void lbt_profile_enable(int on) { lbt::profiler().mode = on < 0 ? 0 : on; }
 void lbt_profile_reset(void)
 {
   auto& p = lbt::profiler();
+  p.collect();
   std::memset(&p.acc, 0, sizeof(p.acc));
 }
 
 void lbt_profile_get(lbt_profile* out)
 {
+  // waits for the calls that returned without synchronising
+  lbt::profiler().collect();
   if (out) *out = lbt::profiler().acc;
 }
 

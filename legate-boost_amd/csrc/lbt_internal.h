@@ -76,18 +76,37 @@ struct ProfSpan {
   hipEvent_t start, stop;
 };
 
+// Per-level counts of one lbt_build_tree call on their way to the host: the call copies them
+// into pinned memory in stream order and does not have to wait for them.
+struct LevelCounts {
+  long long tiles;  // tile count and padding of the device-side record
+  long long instances, built_instances, built_nodes;
+};
+struct ProfLevels {
+  LevelCounts* host;    // pinned, 64 entries
+  hipEvent_t arrived;   // recorded behind the copy
+  int levels;
+  double bytes_per_built_row;
+  double bytes_per_built_node;
+  double root_extra_bytes;
+};
+
 struct Profiler {
   int mode = 0;  // 0 off, 1 every kernel class, 2 the two histogram-stage classes only
   lbt_profile acc{};
-  std::vector<ProfSpan> open;  // spans of the call in flight
+  std::vector<ProfSpan> open;  // spans not yet read back
   std::vector<hipEvent_t> pool;  // events waiting to be reused
+  std::vector<ProfLevels> levels;        // level counts not yet read back
+  std::vector<LevelCounts*> level_pool;  // pinned buffers waiting to be reused
+  // nullptr if no pinned buffer or event can be had
+  ProfLevels* begin_levels(int n_levels, double per_row, double per_node, double root_extra);
   bool wants(int cls) const
   {
     return mode == 1 || (mode == 2 && (cls == LBT_PROF_HISTOGRAM || cls == LBT_PROF_BINNING));
   }
   void begin(int cls, int level, double bytes, hipStream_t s);
   void end(hipStream_t s);
-  void collect();  // after the stream has been synchronised
+  void collect();  // waits for what the recorded events mark, then adds everything up
 };
 Profiler& profiler();
 

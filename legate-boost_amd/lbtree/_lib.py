@@ -104,6 +104,8 @@ def _load():
     lib.lbt_build_tree.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_void_p,
                                    C.c_void_p, C.c_int32, C.c_void_p, C.POINTER(BuildParams), C.c_void_p, C.c_void_p,
                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.POINTER(BuildTaps)]
+    lib.lbt_build_tree_async.restype = C.c_int
+    lib.lbt_build_tree_async.argtypes = lib.lbt_build_tree.argtypes
     lib.lbt_predict.restype = C.c_int
     lib.lbt_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_void_p,
                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t]
@@ -141,7 +143,7 @@ def _load():
 lib = _load()
 
 EXPORTS = [
-    "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_predict",
+    "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_build_tree_async", "lbt_predict",
     "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_profile_enable", "lbt_profile_reset",

@@ -90,7 +90,7 @@ class Tree(BaseModel):
         r = ops.build_tree(
             X, g, h, max_depth=self.max_depth, split_samples=self.split_samples, seed=seed,
             l1_regularization=self.l1_regularization, l2_regularization=self.l2_regularization,
-            min_split_gain=self.min_split_gain, feature_set=feature_set, row_leaf=pred is not None,
+            min_split_gain=self.min_split_gain, feature_set=feature_set, row_leaf=pred is not None, wait=False,
         )
         if pred is not None:
             ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)

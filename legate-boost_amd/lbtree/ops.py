@@ -56,9 +56,10 @@ class BuildResult:
 
 def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0, l2_regularization=1.0,
                min_split_gain=0.0, feature_set=None, dataset_rows=None, row_offset=0, hist_cache_bytes=0,
-               taps=False, taps_levels=False, row_leaf=False):
+               taps=False, taps_levels=False, row_leaf=False, wait=True):
     """BUILD_TREE (legateboost/models/tree.py:104-191). Returns a BuildResult with the five task
-    outputs as CUDA tensors; with taps=True also the observation points."""
+    outputs as CUDA tensors; with taps=True also the observation points. wait=False returns
+    without synchronising the stream (lbt_build_tree_async; not together with taps=True)."""
     X = _check_x(X)
     g = as_device(g, torch.float64)
     h = as_device(h, torch.float64)
@@ -123,7 +124,10 @@ def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0
         tp.level_instances = li.ctypes.data
         tp.level_built_instances = lbi.ctypes.data
         tp.level_built_nodes = lbn.ctypes.data
-    rc = _lib.lib.lbt_build_tree(_stream(), X.data_ptr(), _DT[X.dtype], row_offset, n, f, g.data_ptr(), h.data_ptr(),
+    if taps and not wait:
+        raise _lib.LbtError("the observation points need the synchronising call")
+    call = _lib.lib.lbt_build_tree if wait else _lib.lib.lbt_build_tree_async
+    rc = call(_stream(), X.data_ptr(), _DT[X.dtype], row_offset, n, f, g.data_ptr(), h.data_ptr(),
                                  k, fs.data_ptr() if fs is not None else None, C.byref(prm), r.leaf_value.data_ptr(),
                                  r.feature.data_ptr(), r.split_value.data_ptr(), r.gain.data_ptr(),
                                  r.hessian.data_ptr(), ws.data_ptr() if ws is not None else None,
