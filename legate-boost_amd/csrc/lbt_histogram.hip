@@ -37,6 +37,7 @@
 #include "lbt_internal.h"
 
 #include <algorithm>
+#include <cstring>
 
 namespace lbt {
 namespace {
@@ -1475,6 +1476,69 @@ size_t widest_group(const std::vector<int32_t>& groups, BytesOf bytes_of)
 
 }  // namespace
 
+// The small tables hist_prepare sends to the device (feature groups, record layouts) lie next
+// to each other in the workspace. They are gathered in one pinned block per host thread and
+// sent with one copy: every separate small copy costs about 10 us of the stream's time.
+struct Upload {
+  struct Item {
+    void* dst;
+    const void* src;
+    size_t bytes;
+  };
+  std::vector<Item> items;
+  void add(void* dst, const void* src, size_t bytes)
+  {
+    if (bytes > 0) items.push_back({dst, src, bytes});
+  }
+  // max_slack: bytes that may lie between two tables (the unused tail of a table's
+  // allocation plus the allocator's padding); anything wider means a foreign buffer
+  int send(hipStream_t stream, size_t max_slack)
+  {
+    if (items.empty()) return LBT_OK;
+    std::sort(items.begin(), items.end(), [](const Item& a, const Item& b) { return a.dst < b.dst; });
+    char* const lo = static_cast<char*>(items.front().dst);
+    char* const hi = static_cast<char*>(items.back().dst) + items.back().bytes;
+    bool together  = static_cast<size_t>(hi - lo) <= (size_t(1) << 20);
+    for (size_t i = 1; i < items.size() && together; i++) {
+      const char* prev_end = static_cast<const char*>(items[i - 1].dst) + items[i - 1].bytes;
+      const char* next     = static_cast<const char*>(items[i].dst);
+      together = next >= prev_end && static_cast<size_t>(next - prev_end) <= max_slack;
+    }
+    static thread_local char* stage          = nullptr;
+    static thread_local size_t stage_bytes   = 0;
+    static thread_local hipEvent_t stage_free = nullptr;
+    if (together) {
+      const size_t total = static_cast<size_t>(hi - lo);
+      if (stage_free == nullptr) {
+        if (hipEventCreateWithFlags(&stage_free, hipEventDisableTiming) != hipSuccess) together = false;
+      } else {
+        // the block may still be the source of an earlier call's copy (on another stream)
+        LBT_HIP(hipEventSynchronize(stage_free));
+      }
+      if (together && stage_bytes < total) {
+        if (stage != nullptr) LBT_HIP(hipHostFree(stage));
+        stage       = nullptr;
+        stage_bytes = 0;
+        if (hipHostMalloc(reinterpret_cast<void**>(&stage), total + 4096, hipHostMallocDefault) == hipSuccess)
+          stage_bytes = total + 4096;
+        else
+          together = false;
+      }
+      if (together) {
+        std::memset(stage, 0, total);
+        for (const Item& it : items) std::memcpy(stage + (static_cast<char*>(it.dst) - lo), it.src, it.bytes);
+        LBT_HIP(hipMemcpyAsync(lo, stage, total, hipMemcpyHostToDevice, stream));
+        LBT_HIP(hipEventRecord(stage_free, stream));
+        items.clear();
+        return LBT_OK;
+      }
+    }
+    for (const Item& it : items) LBT_HIP(hipMemcpyAsync(it.dst, it.src, it.bytes, hipMemcpyHostToDevice, stream));
+    items.clear();
+    return LBT_OK;
+  }
+};
+
 int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, int64_t n_rows,
                  const std::vector<int32_t>& rp, const void* proposals, const int32_t* row_pointers,
                  const void* X)
@@ -1537,7 +1601,8 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   hs.n_sgroups = static_cast<int>(sgroups.size()) - 1;
   hs.lds_bytes = (search_lds + (cached ? kProbeSlack * elem : 0) + 15) & ~size_t(15);
   hs.rpp       = rows_per_pass(sgroups, vec);
-  LBT_HIP(hipMemcpyAsync(hs.sgroups, sgroups.data(), sizeof(int32_t) * sgroups.size(), hipMemcpyHostToDevice, stream));
+  Upload up;
+  up.add(hs.sgroups, sgroups.data(), sizeof(int32_t) * sgroups.size());
 
   base.assign(F, 0);
   stride.assign(F, 0);
@@ -1562,7 +1627,7 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     hs.partial_stride = static_cast<int>(blds / 8);  // bins of the widest group
     if (hs.partial_stride > kPartialStrideMax) hs.partials = nullptr;
     hs.brpp       = rows_per_pass(groups, hs.bvec);
-    LBT_HIP(hipMemcpyAsync(hs.groups, groups.data(), sizeof(int32_t) * groups.size(), hipMemcpyHostToDevice, stream));
+    up.add(hs.groups, groups.data(), sizeof(int32_t) * groups.size());
     // record layout of every histogram group
     const int chunk = hs.bvec * hs.bin_bytes;  // bytes a lane of the histogram kernel loads
     // The records of a row lie side by side ([row][group]): the binning pass, whose lanes hold a
@@ -1600,11 +1665,13 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       set_error("bin cache of %lld bytes exceeds the workspace share", static_cast<long long>(at));
       return LBT_ERR_WORKSPACE;
     }
-    LBT_HIP(hipMemcpyAsync(hs.rec, rec.data(), sizeof(RecInfo) * rec.size(), hipMemcpyHostToDevice, stream));
-    LBT_HIP(hipMemcpyAsync(hs.bin_base, base.data(), sizeof(int64_t) * F, hipMemcpyHostToDevice, stream));
-    LBT_HIP(hipMemcpyAsync(hs.bin_stride, stride.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
-    LBT_HIP(hipMemcpyAsync(hs.bin_tail, tail.data(), sizeof(int32_t) * F, hipMemcpyHostToDevice, stream));
+    up.add(hs.rec, rec.data(), sizeof(RecInfo) * rec.size());
+    up.add(hs.bin_base, base.data(), sizeof(int64_t) * F);
+    up.add(hs.bin_stride, stride.data(), sizeof(int32_t) * F);
+    up.add(hs.bin_tail, tail.data(), sizeof(int32_t) * F);
   }
+  // the tables are allocated one behind the other, each with room for F entries of up to 24 bytes
+  LBT_TRY(up.send(stream, static_cast<size_t>(F) * sizeof(RecInfo) + 512));
   ProfScope ps(LBT_PROF_PROPOSALS, stream);
   if (is_f64)
     build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,
