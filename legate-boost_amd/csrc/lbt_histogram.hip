@@ -1261,35 +1261,23 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
 }
 
 template <typename BinT, int BV, bool kEmbed, bool kRoot>
-int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid)
+int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
+                     const PartialSink& sink)
 {
-  PartialSink sink{hs.partials, hs.partial_lists, hs.partial_list_count, hs.partial_count, 0, hs.partial_stride};
-  if (hs.partials != nullptr && static_cast<int64_t>(a.w.n_nodes) * a.w.n_gk <= kPartialMaxLists)
-    sink.slots = hs.partial_slots;
   static bool attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
     kRoot && a.w.n_gk > 1 && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr, sink);
-  if (sink.slots > 0) {
-    // the stride is the widest group in bins; near the root, where few lists are long, the slots of
-    // a list are dealt to several workgroups
-    const int lists      = a.w.n_nodes * a.w.n_gk;
-    const int bin_chunks = (sink.stride + kHistThreads - 1) / kHistThreads;
-    const int split      = std::max(1, std::min(16, 256 / (lists * bin_chunks)));
-    dim3 rgrid(static_cast<unsigned>(bin_chunks), static_cast<unsigned>(lists), static_cast<unsigned>(split));
-    reduce_partials_kernel<<<rgrid, kHistThreads, 0, stream>>>(sink, a.K, a.w.n_gk / a.K, a.groups, a.row_pointers,
-                                                               a.hist, a.w.level_first + a.w.j0);
-  }
   return LBT_OK;
 }
 template <typename BinT, int BV, bool kEmbed>
 int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
-                  bool root)
+                  bool root, const PartialSink& sink)
 {
-  if (root) return launch_binned_as<BinT, BV, kEmbed, true>(stream, hs, a, b, grid);
-  return launch_binned_as<BinT, BV, kEmbed, false>(stream, hs, a, b, grid);
+  if (root) return launch_binned_as<BinT, BV, kEmbed, true>(stream, hs, a, b, grid, sink);
+  return launch_binned_as<BinT, BV, kEmbed, false>(stream, hs, a, b, grid, sink);
 }
 
 // As many resident workgroups as the LDS allows per CU; row-tile ranges come in multiples
@@ -1380,7 +1368,6 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
                                     hs.tiles, root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr,
                                     use_cache ? hs.partial_count : nullptr, hs.partial_list_count);
   }
-  ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   if (use_cache) {
     BinnedArgs a;
     a.w            = w;
@@ -1389,12 +1376,35 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     a.row_pointers = b.row_pointers;
     a.groups       = hs.groups;
     a.hist         = b.hist;
-    if (hs.bin_bytes == 1)
-      return hs.embed ? launch_binned<uint8_t, 16, true>(stream, hs, a, b, grid, root)
-                      : launch_binned<uint8_t, 16, false>(stream, hs, a, b, grid, root);
-    return hs.embed ? launch_binned<uint16_t, 4, true>(stream, hs, a, b, grid, root)
-                    : launch_binned<uint16_t, 4, false>(stream, hs, a, b, grid, root);
+    PartialSink sink{hs.partials, hs.partial_lists, hs.partial_list_count, hs.partial_count, 0, hs.partial_stride};
+    if (hs.partials != nullptr && static_cast<int64_t>(w.n_nodes) * w.n_gk <= kPartialMaxLists)
+      sink.slots = hs.partial_slots;
+    {
+      ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
+      int rc;
+      if (hs.bin_bytes == 1)
+        rc = hs.embed ? launch_binned<uint8_t, 16, true>(stream, hs, a, b, grid, root, sink)
+                      : launch_binned<uint8_t, 16, false>(stream, hs, a, b, grid, root, sink);
+      else
+        rc = hs.embed ? launch_binned<uint16_t, 4, true>(stream, hs, a, b, grid, root, sink)
+                      : launch_binned<uint16_t, 4, false>(stream, hs, a, b, grid, root, sink);
+      LBT_TRY(rc);
+    }
+    if (sink.slots > 0) {
+      // timed with the scan, which is the other pass over the finished histograms
+      ProfScope ps(LBT_PROF_SCAN, stream);
+      // the stride is the widest group in bins; near the root, where few lists are long, the slots of
+      // a list are dealt to several workgroups
+      const int lists      = w.n_nodes * w.n_gk;
+      const int bin_chunks = (sink.stride + kHistThreads - 1) / kHistThreads;
+      const int split      = std::max(1, std::min(16, 256 / (lists * bin_chunks)));
+      dim3 rgrid(static_cast<unsigned>(bin_chunks), static_cast<unsigned>(lists), static_cast<unsigned>(split));
+      reduce_partials_kernel<<<rgrid, kHistThreads, 0, stream>>>(sink, a.K, w.n_gk / a.K, a.groups, a.row_pointers, a.hist,
+                                                                 w.level_first + w.j0);
+    }
+    return LBT_OK;
   }
+  ProfScope ps(LBT_PROF_HISTOGRAM, stream, 0.0, depth);
   HistArgs<T> a;
   a.w            = w;
   a.F            = b.F;
