@@ -343,6 +343,29 @@ def test_gather_rows_matches_oracle(dtype):
     assert ops.gather_rows(X, (), row_offset=0).shape == (0, 17)
 
 
+def test_async_build_gives_the_same_tree_and_defers_the_profile():
+    from lbtree import _lib, ops
+
+    X, g, h = _problem(77, 40000, 12, 2)
+    kw = dict(max_depth=6, split_samples=64, seed=11, row_leaf=True)
+    a = ops.build_tree(X, g, h, **kw)
+    _lib.profile_reset()
+    _lib.profile_enable(1)
+    try:
+        b = [ops.build_tree(X, g, h, wait=False, **kw) for _ in range(3)]  # queued back to back on one workspace
+        prof = _lib.profile_get()  # waits for the three calls
+    finally:
+        _lib.profile_enable(0)
+    for r in b:
+        for name in ["leaf_value", "feature", "split_value", "gain", "hessian", "row_leaf"]:
+            assert torch.equal(getattr(a, name), getattr(r, name)), name
+    assert prof["histogram"]["launches"] == 3 * 6 and prof["binning"]["launches"] == 3
+    assert len(prof["levels"]) == 6 and prof["levels"][0]["instances"] == 3 * 40000
+    assert all(lv["built_instances"] <= lv["instances"] for lv in prof["levels"])
+    with pytest.raises(_lib.LbtError):
+        ops.build_tree(X, g, h, max_depth=3, split_samples=16, seed=1, taps=True, wait=False)
+
+
 def test_two_runs_are_bit_identical():
     import gpu_util as gu
 
