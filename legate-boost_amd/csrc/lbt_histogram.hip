@@ -1026,6 +1026,7 @@ __global__ void __launch_bounds__(kHistThreads)
   int c_base[BV];
 #pragma unroll
   for (int v = 0; v < BV; v++) c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
+  const int nv = min(BV, max(0, gs - fl));  // features this lane really has
   const unsigned long long max_abs = qstats[0];
   const int n_tiles = meta->n_tiles;
   const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
@@ -1185,8 +1186,10 @@ __global__ void __launch_bounds__(kHistThreads)
           int rel[BV];
           unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
-          // features past the group end read zero bytes of the record: spare slot
-          for (int v = 0; v < BV; v++) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
+          // a lane whose 16 bins reach past the group end leaves those out: an atomic costs by
+          // the lanes that take part in it
+          for (int v = 0; v < BV; v++)
+            if (v < nv) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
         }
       }
     } else {
