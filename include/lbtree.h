@@ -125,6 +125,42 @@ int lbt_build_tree_async(void* stream, const void* X, int32_t x_dtype, int64_t r
                          double* leaf, int32_t* feature, double* split, double* gain, double* hessian,
                          void* workspace, size_t workspace_bytes, lbt_build_taps* taps);
 
+/*
+ * Two stages of BuildTreeTask on their own, so that each can be checked and timed alone.
+ * lbt_build_tree runs the same kernels.
+ *
+ * SelectSplitSamples (build_tree.cu:867-964): split_samples rows drawn with minstd_rand from
+ * [0, dataset_rows), their values gathered per feature (rows outside
+ * [row_offset, row_offset + n_rows) contribute 0, build_tree.cu:889-899), sorted, made unique,
+ * the last proposal of every feature replaced by +inf.
+ *   proposals     device, X dtype, [n_features * split_samples]; the first row_pointers[n_features]
+ *                 entries are written, feature by feature
+ *   row_pointers  device int32 [n_features + 1]
+ *   workspace     device scratch of lbt_select_split_samples_workspace_bytes(...)
+ * Enqueues on the stream, does not wait.
+ */
+size_t lbt_select_split_samples_workspace_bytes(int32_t n_features, int32_t split_samples, int32_t x_dtype);
+int lbt_select_split_samples(void* stream, const void* X, int32_t x_dtype, int64_t row_offset, int64_t n_rows,
+                             int32_t n_features, int32_t split_samples, int32_t seed, int64_t dataset_rows,
+                             void* proposals, int32_t* row_pointers, void* workspace, size_t workspace_bytes);
+
+/*
+ * GradientQuantiser and reduce_base_sums (build_tree.cu:51-140, :168-204): scale = (2^31 - 1) / sum|.|
+ * over all entries of g and of h, one stochastic rounding per (row, output) seeded by
+ * hash_combine(seed, row_offset + row, output) (build_tree.cu:143-165), and the sums of the
+ * rounded pairs per output.
+ *   quantised  device int32 [n_rows][n_outputs][2] (grad, hess)
+ *   root_sums  device int64 [n_outputs][2]
+ *   scales     device double [4]: scale.grad, scale.hess, 1/scale.grad, 1/scale.hess
+ *   workspace  device scratch of lbt_quantise_gradients_workspace_bytes(...)
+ * Enqueues on the stream, does not wait. A rounded value that does not fit 32 bits is
+ * stored truncated here; lbt_build_tree reports it as LBT_ERR_UNSUPPORTED.
+ */
+size_t lbt_quantise_gradients_workspace_bytes(int64_t n_rows, int32_t n_outputs);
+int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64_t n_rows, int32_t n_outputs,
+                           int64_t row_offset, int32_t seed, int32_t* quantised, int64_t* root_sums, double* scales,
+                           void* workspace, size_t workspace_bytes);
+
 /* Device scratch for lbt_predict: room for the ensemble packed into one node array and one
  * leaf array (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
 size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype);

@@ -1319,6 +1319,60 @@ int host_mirror(int F, HostMirror** out)
   return LBT_OK;
 }
 
+// SelectSplitSamples (build_tree.cu:867-964): gather, sort and unique per feature, row pointers,
+// compaction. draft and uniq hold F * S values of T each, counts F and bin_feature F * S ints.
+template <typename T>
+int run_split_samples(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F, int S, int32_t seed,
+                      int64_t dataset_rows, T* draft, T* uniq, int32_t* counts, int32_t* row_pointers, T* proposals,
+                      int32_t* bin_feature)
+{
+  auto blocks = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+  gather_samples_kernel<T><<<blocks(static_cast<int64_t>(F) * S, kThreads), kThreads, 0, stream>>>(
+    X, row_offset, N, F, S, seed, dataset_rows, draft);
+  int P = 1;
+  while (P < S) P <<= 1;
+  if (P < 2) P = 2;
+  sort_unique_kernel<T><<<F, kThreads, P * sizeof(typename KeyOf<T>::type), stream>>>(draft, S, P, uniq, counts);
+  row_pointers_kernel<<<1, 64, 0, stream>>>(counts, F, row_pointers);
+  compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(uniq, S, row_pointers, proposals, bin_feature);
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
+// GradientQuantiser and reduce_base_sums (build_tree.cu:51-140, :168-204): the two absolute sums
+// in a fixed order, the scales, one rounding per (row, output), and the sums of the rounded pairs
+// added to root_sums[k] (which the caller has cleared). part_a/part_b: two levels of partial sums.
+int run_quantiser(hipStream_t stream, const double* g, const double* h, int64_t N, int K, int64_t row_offset,
+                  int32_t seed, double* const (&part_a)[2], double* const (&part_b)[2], double* scales,
+                  unsigned long long* qstats, int2* qgh, I64Pair* root_sums)
+{
+  auto blocks = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+  int64_t n = N * K;
+  int64_t m = (n + 4095) / 4096;
+  abs_sum_level_kernel<true><<<static_cast<unsigned>(m), kThreads, 0, stream>>>(g, h, n, part_a[0], part_b[0]);
+  int cur = 0;
+  while (m > 1) {
+    int64_t m2 = (m + 4095) / 4096;
+    abs_sum_level_kernel<false><<<static_cast<unsigned>(m2), kThreads, 0, stream>>>(part_a[cur], part_b[cur], m,
+                                                                                     part_a[cur ^ 1], part_b[cur ^ 1]);
+    cur ^= 1;
+    m = m2;
+  }
+  scales_kernel<<<1, 64, 0, stream>>>(part_a[cur], part_b[cur], scales, qstats);
+  if (K > 1 && K <= kQuantiseFlatMaxK) {
+    const unsigned gx =
+      std::max<unsigned>(std::min<unsigned>(blocks(N * K, kThreads), 2048u), blocks(K, kThreads));
+    quantise_flat_kernel<<<gx, kThreads, 2 * K * sizeof(unsigned long long), stream>>>(
+      g, h, N, K, row_offset, static_cast<int64_t>(seed), scales, qgh, root_sums, qstats);
+  } else {
+    dim3 grid(std::min<unsigned>(blocks(N, kThreads), 2048u), K);
+    quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(seed), scales, qgh,
+                                                   root_sums, qstats);
+  }
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
 template <typename T>
 int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F,
                     const double* g, const double* h, int K, const uint8_t* feature_set,
@@ -1342,46 +1396,17 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   int32_t* const rp_here = hm->pinned + 4;
   {
     ProfScope ps(LBT_PROF_PROPOSALS, stream);
-    T* draft = static_cast<T*>(L.draft);
-    T* uniq  = static_cast<T*>(L.uniq);
-    gather_samples_kernel<T><<<blocks(static_cast<int64_t>(F) * S, kThreads), kThreads, 0, stream>>>(
-      X, row_offset, N, F, S, prm.seed, prm.dataset_rows, draft);
-    int P = 1;
-    while (P < S) P <<= 1;
-    if (P < 2) P = 2;
-    sort_unique_kernel<T><<<F, kThreads, P * sizeof(typename KeyOf<T>::type), stream>>>(
-      draft, S, P, uniq, L.counts);
-    row_pointers_kernel<<<1, 64, 0, stream>>>(L.counts, F, L.row_pointers);
-    compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(
-      uniq, S, L.row_pointers, static_cast<T*>(L.proposals), L.bin_feature);
+    LBT_TRY(run_split_samples<T>(stream, X, row_offset, N, F, S, prm.seed, prm.dataset_rows, static_cast<T*>(L.draft),
+                                 static_cast<T*>(L.uniq), L.counts, L.row_pointers, static_cast<T*>(L.proposals),
+                                 L.bin_feature));
     LBT_HIP(hipMemcpyAsync(rp_here, L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
     LBT_HIP(hipEventRecord(hm->counts_here, stream));
   }
   // ---- quantiser
   {
     ProfScope ps(LBT_PROF_QUANTISE, stream, static_cast<double>(N) * K * (16 + 16 + 8));
-    int64_t n = N * K;
-    int64_t m = (n + 4095) / 4096;
-    abs_sum_level_kernel<true><<<static_cast<unsigned>(m), kThreads, 0, stream>>>(g, h, n, L.part_a[0], L.part_b[0]);
-    int cur = 0;
-    while (m > 1) {
-      int64_t m2 = (m + 4095) / 4096;
-      abs_sum_level_kernel<false><<<static_cast<unsigned>(m2), kThreads, 0, stream>>>(
-        L.part_a[cur], L.part_b[cur], m, L.part_a[cur ^ 1], L.part_b[cur ^ 1]);
-      cur ^= 1;
-      m = m2;
-    }
-    scales_kernel<<<1, 64, 0, stream>>>(L.part_a[cur], L.part_b[cur], L.scales, L.qstats);
-    if (K > 1 && K <= kQuantiseFlatMaxK) {
-      const unsigned gx = std::max<unsigned>(std::min<unsigned>(blocks(N * K, kThreads), 2048u),
-                                             blocks(K, kThreads));
-      quantise_flat_kernel<<<gx, kThreads, 2 * K * sizeof(unsigned long long), stream>>>(
-        g, h, N, K, row_offset, static_cast<int64_t>(prm.seed), L.scales, L.qgh, L.node_sums, L.qstats);
-    } else {
-      dim3 grid(std::min<unsigned>(blocks(N, kThreads), 2048u), K);
-      quantise_kernel<<<grid, kThreads, 0, stream>>>(g, h, N, K, row_offset, static_cast<int64_t>(prm.seed),
-                                                     L.scales, L.qgh, L.node_sums, L.qstats);
-    }
+    LBT_TRY(run_quantiser(stream, g, h, N, K, row_offset, prm.seed, L.part_a, L.part_b, L.scales, L.qstats, L.qgh,
+                          L.node_sums));
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization);
   }
@@ -1656,6 +1681,53 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
 }  // namespace
 }  // namespace lbt
 
+namespace {
+
+struct SampleScratch {
+  char* draft;
+  char* uniq;
+  int32_t* counts;
+  int32_t* bin_feature;
+};
+void make_sample_scratch(lbt::Arena& ar, SampleScratch& w, int F, int S, size_t elem)
+{
+  w.draft       = ar.take<char>(static_cast<size_t>(F) * S * elem);
+  w.uniq        = ar.take<char>(static_cast<size_t>(F) * S * elem);
+  w.counts      = ar.take<int32_t>(F);
+  w.bin_feature = ar.take<int32_t>(static_cast<size_t>(F) * S);
+}
+
+struct QuantiserScratch {
+  double* part_a[2];
+  double* part_b[2];
+  unsigned long long* qstats;
+};
+void make_quantiser_scratch(lbt::Arena& ar, QuantiserScratch& w, int64_t N, int K)
+{
+  int64_t n_chunks = (N * K + 4095) / 4096;
+  for (int i = 0; i < 2; i++) {
+    w.part_a[i] = ar.take<double>(n_chunks);
+    w.part_b[i] = ar.take<double>(n_chunks);
+    n_chunks    = (n_chunks + 4095) / 4096;
+  }
+  w.qstats = ar.take<unsigned long long>(2);
+}
+
+int arena_over(lbt::Arena& ar, void* workspace, size_t workspace_bytes)
+{
+  if (workspace == nullptr) {
+    lbt::set_error("workspace is null");
+    return LBT_ERR_WORKSPACE;
+  }
+  const uintptr_t raw     = reinterpret_cast<uintptr_t>(workspace);
+  const uintptr_t aligned = (raw + 255) & ~uintptr_t(255);
+  ar.base                 = reinterpret_cast<char*>(aligned);
+  ar.cap                  = workspace_bytes > (aligned - raw) ? workspace_bytes - (aligned - raw) : 0;
+  return LBT_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_t n_outputs,
@@ -1715,6 +1787,82 @@ static int build_tree_entry(void* stream, const void* X, int32_t x_dtype, int64_
     lbt::profiler().collect();
   }
   return rc;
+}
+
+size_t lbt_select_split_samples_workspace_bytes(int32_t n_features, int32_t split_samples, int32_t x_dtype)
+{
+  if (n_features < 1 || split_samples < 1 || split_samples > LBT_MAX_SPLIT_SAMPLES) return 0;
+  if (x_dtype != LBT_F32 && x_dtype != LBT_F64) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  SampleScratch w;
+  make_sample_scratch(ar, w, n_features, split_samples, x_dtype == LBT_F64 ? 8 : 4);
+  return ar.used + 256;
+}
+
+int lbt_select_split_samples(void* stream, const void* X, int32_t x_dtype, int64_t row_offset, int64_t n_rows,
+                             int32_t n_features, int32_t split_samples, int32_t seed, int64_t dataset_rows,
+                             void* proposals, int32_t* row_pointers, void* workspace, size_t workspace_bytes)
+{
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(n_rows >= 0 && n_rows < 2147483647LL && n_features >= 1, "bad shape");
+  LBT_REQUIRE(split_samples >= 1 && split_samples <= LBT_MAX_SPLIT_SAMPLES, "split_samples must be in [1, %d]",
+              LBT_MAX_SPLIT_SAMPLES);
+  LBT_REQUIRE(dataset_rows >= 1 && row_offset >= 0, "dataset_rows must be positive, row_offset not negative");
+  LBT_REQUIRE((X || n_rows == 0) && proposals && row_pointers, "null input or output pointer");
+  lbt::Arena ar;
+  LBT_TRY(arena_over(ar, workspace, workspace_bytes));
+  SampleScratch w;
+  make_sample_scratch(ar, w, n_features, split_samples, x_dtype == LBT_F64 ? 8 : 4);
+  if (ar.failed) {
+    lbt::set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  lbt::ProfScope ps(LBT_PROF_PROPOSALS, s);
+  if (x_dtype == LBT_F32)
+    return lbt::run_split_samples<float>(s, static_cast<const float*>(X), row_offset, n_rows, n_features, split_samples,
+                                         seed, dataset_rows, reinterpret_cast<float*>(w.draft),
+                                         reinterpret_cast<float*>(w.uniq), w.counts, row_pointers,
+                                         static_cast<float*>(proposals), w.bin_feature);
+  return lbt::run_split_samples<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, split_samples,
+                                        seed, dataset_rows, reinterpret_cast<double*>(w.draft),
+                                        reinterpret_cast<double*>(w.uniq), w.counts, row_pointers,
+                                        static_cast<double*>(proposals), w.bin_feature);
+}
+
+size_t lbt_quantise_gradients_workspace_bytes(int64_t n_rows, int32_t n_outputs)
+{
+  if (n_rows < 1 || n_outputs < 1 || n_rows >= 2147483647LL) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  QuantiserScratch w;
+  make_quantiser_scratch(ar, w, n_rows, n_outputs);
+  return ar.used + 256;
+}
+
+int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64_t n_rows, int32_t n_outputs,
+                           int64_t row_offset, int32_t seed, int32_t* quantised, int64_t* root_sums, double* scales,
+                           void* workspace, size_t workspace_bytes)
+{
+  LBT_REQUIRE(n_rows >= 1 && n_rows < 2147483647LL && n_outputs >= 1 && n_outputs <= 65535, "bad shape");
+  LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
+  LBT_REQUIRE(g && h && quantised && root_sums && scales, "null input or output pointer");
+  lbt::Arena ar;
+  LBT_TRY(arena_over(ar, workspace, workspace_bytes));
+  QuantiserScratch w;
+  make_quantiser_scratch(ar, w, n_rows, n_outputs);
+  if (ar.failed) {
+    lbt::set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  lbt::ProfScope ps(LBT_PROF_QUANTISE, s, static_cast<double>(n_rows) * n_outputs * (16 + 16 + 8));
+  // the sums are added to: clear them with a kernel (a memset node would not replay in a captured graph)
+  static_assert(sizeof(lbt::I64Pair) == 16, "root sums are cleared in 16-byte units");
+  lbt::zero_kernel<<<1, lbt::kThreads, 0, s>>>(reinterpret_cast<uint4*>(root_sums), n_outputs);
+  return lbt::run_quantiser(s, g, h, n_rows, n_outputs, row_offset, seed, w.part_a, w.part_b, scales, w.qstats,
+                            reinterpret_cast<int2*>(quantised), reinterpret_cast<lbt::I64Pair*>(root_sums));
 }
 
 int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,

@@ -132,6 +132,17 @@ def _load():
     lib.lbt_gather_rows.restype = C.c_int
     lib.lbt_gather_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_void_p,
                                     C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.lbt_select_split_samples_workspace_bytes.restype = C.c_size_t
+    lib.lbt_select_split_samples_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+    lib.lbt_select_split_samples.restype = C.c_int
+    lib.lbt_select_split_samples.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int32,
+                                             C.c_int32, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.c_size_t]
+    lib.lbt_quantise_gradients_workspace_bytes.restype = C.c_size_t
+    lib.lbt_quantise_gradients_workspace_bytes.argtypes = [C.c_int64, C.c_int32]
+    lib.lbt_quantise_gradients.restype = C.c_int
+    lib.lbt_quantise_gradients.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64,
+                                           C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.lbt_profile_enable.restype = None
     lib.lbt_profile_enable.argtypes = [C.c_int]
     lib.lbt_profile_reset.restype = None
@@ -146,7 +157,8 @@ EXPORTS = [
     "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_build_tree_async", "lbt_predict",
     "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
-    "lbt_gather_rows", "lbt_profile_enable", "lbt_profile_reset",
+    "lbt_gather_rows", "lbt_select_split_samples_workspace_bytes", "lbt_select_split_samples",
+    "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",
 ]
 

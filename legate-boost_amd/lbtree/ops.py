@@ -317,3 +317,39 @@ def gather_rows(X, samples, row_offset=0):
     if on_host:
         torch.cuda.current_stream().synchronize()  # the host array is read by the copy on the stream
     return out
+
+
+def select_split_samples(X, split_samples, seed, dataset_rows=None, row_offset=0):
+    """SelectSplitSamples on its own (build_tree.cu:867-964): returns (proposals, row_pointers),
+    the proposals of feature f at proposals[row_pointers[f]:row_pointers[f + 1]], ascending,
+    the last one +inf."""
+    X = _check_x(X)
+    n, f = X.shape
+    dt = _DT[X.dtype]
+    ws = torch.empty(_lib.lib.lbt_select_split_samples_workspace_bytes(f, split_samples, dt), dtype=torch.uint8,
+                     device=X.device)
+    props = torch.empty(f * split_samples, dtype=X.dtype, device=X.device)
+    rp = torch.empty(f + 1, dtype=torch.int32, device=X.device)
+    rc = _lib.lib.lbt_select_split_samples(_stream(), X.data_ptr(), dt, row_offset, n, f, split_samples, seed,
+                                           n if dataset_rows is None else dataset_rows, props.data_ptr(),
+                                           rp.data_ptr(), ws.data_ptr(), ws.numel())
+    _lib.check(rc)
+    return props[: int(rp[-1])], rp
+
+
+def quantise_gradients(g, h, seed, row_offset=0):
+    """GradientQuantiser and the root sums on their own (build_tree.cu:51-140, :168-204): returns
+    (quantised int32 [n][K][2], root_sums int64 [K][2], scales f64 [4])."""
+    g = g.contiguous()
+    h = h.contiguous()
+    if g.dtype != torch.float64 or h.dtype != torch.float64 or g.shape != h.shape or g.dim() != 2:
+        raise ValueError("g and h must be float64 [n_rows][n_outputs] of the same shape")
+    n, k = g.shape
+    ws = torch.empty(_lib.lib.lbt_quantise_gradients_workspace_bytes(n, k), dtype=torch.uint8, device=g.device)
+    q = torch.empty((n, k, 2), dtype=torch.int32, device=g.device)
+    sums = torch.empty((k, 2), dtype=torch.int64, device=g.device)
+    scales = torch.empty(4, dtype=torch.float64, device=g.device)
+    rc = _lib.lib.lbt_quantise_gradients(_stream(), g.data_ptr(), h.data_ptr(), n, k, row_offset, seed, q.data_ptr(),
+                                         sums.data_ptr(), scales.data_ptr(), ws.data_ptr(), ws.numel())
+    _lib.check(rc)
+    return q, sums, scales

@@ -87,6 +87,19 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert _lib.lib.lbt_gather_rows(None, one, 3, 0, 10, 2, one, 4, 0, None, one) == -1
     rc = _lib.lib.lbt_gather_rows(None, one, _lib.LBT_F32, 0, 10, 2, one, 4, 1, None, one)
     assert rc == -1 and b"staging" in _lib.lib.lbt_last_error()
+    q = _lib.lib.lbt_select_split_samples_workspace_bytes
+    assert 0 < q(4, 16, _lib.LBT_F32) <= q(4, 16, _lib.LBT_F64) and q(4, 4096, _lib.LBT_F32) == 0
+    sel = _lib.lib.lbt_select_split_samples
+    assert sel(None, one, _lib.LBT_F32, 0, 10, 2, 4096, 1, 10, one, one, one, 1 << 20) == -1
+    assert b"split_samples" in _lib.lib.lbt_last_error()
+    assert sel(None, one, _lib.LBT_F32, 0, 10, 2, 16, 1, 0, one, one, one, 1 << 20) == -1
+    assert sel(None, one, _lib.LBT_F32, 0, 10, 2, 16, 1, 10, one, one, one, 8) == -3
+    assert _lib.lib.lbt_quantise_gradients_workspace_bytes(1000, 2) > 0
+    assert _lib.lib.lbt_quantise_gradients_workspace_bytes(0, 2) == 0
+    qg = _lib.lib.lbt_quantise_gradients
+    assert qg(None, one, one, 10, 0, 0, 1, one, one, one, one, 1 << 20) == -1
+    assert qg(None, one, one, 10, 1, 0, 1, one, None, one, one, 1 << 20) == -1
+    assert qg(None, one, one, 10, 1, 0, 1, one, one, one, one, 8) == -3
     with pytest.raises(_lib.LbtError):
         _lib.check(rc)
 

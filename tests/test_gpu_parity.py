@@ -388,3 +388,56 @@ def test_errors_surface_as_exceptions():
         ops.build_tree(X.astype(np.float16), g, g, max_depth=2, split_samples=16, seed=0)
     with pytest.raises(_lib.LbtError):
         ops.build_tree(X, g[:5], g[:5], max_depth=2, split_samples=16, seed=0)
+
+
+@pytest.mark.parametrize("n,f,s,dtype,offset,total", [
+    (5000, 7, 64, np.float32, 0, None),
+    (300, 3, 256, np.float64, 0, None),      # more samples than rows: duplicates collapse
+    (4000, 12, 2048, np.float32, 0, None),
+    (1000, 5, 32, np.float32, 2500, 6000),   # a shard in the middle of a larger dataset: other rows give 0
+    (1, 2, 8, np.float64, 0, None),
+])
+def test_select_split_samples_stage(n, f, s, dtype, offset, total):
+    """The stage on its own against the oracle's restatement of SelectSplitSamples
+    (build_tree.cu:867-964): proposals bit for bit, and the same ones the whole build uses."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    X, g, h = _problem(n + f, n, f, 1, dtype)
+    props, rp = ops.select_split_samples(torch.from_numpy(X).cuda(), s, 77, dataset_rows=total, row_offset=offset)
+    want, want_rp = orc.split_proposals(X, 77, s, dataset_rows=total, row_offset=offset)
+    assert np.array_equal(gu.cpu(rp), want_rp)
+    assert np.array_equal(gu.cpu(props).view(np.uint8), want.view(np.uint8))
+    # ascending inside a feature, +inf last
+    pr, r = gu.cpu(props), gu.cpu(rp)
+    for j in range(f):
+        seg = pr[r[j]:r[j + 1]]
+        assert seg.size >= 1 and np.isinf(seg[-1]) and np.all(np.diff(seg) > 0)
+    if offset == 0 and total is None:
+        t = ops.build_tree(torch.from_numpy(X).cuda(), torch.from_numpy(g).cuda(), torch.from_numpy(h).cuda(),
+                           max_depth=1, split_samples=s, seed=77, taps=True)
+        assert np.array_equal(gu.cpu(t.row_pointers), gu.cpu(rp))
+        assert np.array_equal(gu.cpu(t.proposals).view(np.uint8), pr.view(np.uint8))
+
+
+@pytest.mark.parametrize("n,k,offset", [(5000, 1, 0), (3000, 3, 0), (700, 8, 123456), (1, 1, 0), (9000, 2, 7)])
+def test_quantise_gradients_stage(n, k, offset):
+    """The quantiser on its own against the oracle (build_tree.cu:51-140, :143-165, :168-204): the
+    scales from the absolute sums in the fixed order, every rounded pair and the root sums."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(n + k)
+    g = rs.randn(n, k) * np.exp(rs.randn(n, 1))
+    h = rs.rand(n, k) + 1e-3
+    q, sums, sc = ops.quantise_gradients(torch.from_numpy(g).cuda(), torch.from_numpy(h).cuda(), 4242,
+                                         row_offset=offset)
+    want_sc = orc.scales(orc.abs_sums(g, h))
+    assert np.array_equal(gu.cpu(sc), want_sc)
+    want = orc.quantise_all(g, h, 4242, want_sc, row_offset=offset)
+    assert np.array_equal(gu.cpu(q).astype(np.int64), want)
+    assert np.array_equal(gu.cpu(sums), want.sum(axis=0))
+    # each rounded value is within one unit of the scaled input
+    assert np.all(np.abs(want[:, :, 0] - g * want_sc[0]) < 1.0)
