@@ -441,3 +441,44 @@ def test_quantise_gradients_stage(n, k, offset):
     assert np.array_equal(gu.cpu(sums), want.sum(axis=0))
     # each rounded value is within one unit of the scaled input
     assert np.all(np.abs(want[:, :, 0] - g * want_sc[0]) < 1.0)
+
+
+def test_property_sweep_against_the_oracle():
+    """Drawn cases in the ranges of the reference's property tests (test_with_hypothesis.py:26-40,
+    148-168: depth 1..8, split_samples 1..500, both dtypes, sample weights, feature fractions), plus
+    what the histogram layouts depend on (feature counts either side of a group, two-byte bins, small
+    histogram budgets, skewed and low-cardinality columns). Every case is printed before it runs."""
+    from hypothesis import HealthCheck, given, settings, strategies as st
+    import gpu_util as gu
+
+    @settings(max_examples=60, deadline=None, derandomize=True, database=None,
+              suppress_health_check=list(HealthCheck))
+    @given(n=st.sampled_from([1, 37, 600, 4000, 25000]), f=st.sampled_from([1, 2, 5, 17, 64, 65, 130]),
+           k=st.sampled_from([1, 1, 2, 4]), depth=st.integers(1, 8), s=st.integers(1, 500),
+           f64=st.booleans(), kind=st.integers(0, 3), budget=st.sampled_from([0, 0, 150000, 4000000]),
+           frac=st.sampled_from([1.0, 1.0, 0.5]), weighted=st.booleans(), seed=st.integers(0, 2**31 - 1))
+    def run(n, f, k, depth, s, f64, kind, budget, frac, weighted, seed):
+        print("case", dict(n=n, f=f, k=k, depth=depth, s=s, f64=f64, kind=kind, budget=budget, frac=frac,
+                           weighted=weighted, seed=seed), flush=True)
+        rs = np.random.RandomState(seed % 100003)
+        if n * f > 1_500_000:
+            n = 1_500_000 // f
+        X = rs.randn(n, f).astype(np.float64 if f64 else np.float32)
+        if kind == 1:
+            X[:, 0] = rs.randint(0, 3, n)             # low cardinality
+        elif kind == 2:
+            X = np.exp(3 * X).astype(X.dtype)         # skewed
+        elif kind == 3:
+            X[: n // 2] = np.sort(X[: n // 2], axis=0)  # partly sorted: nodes become row ranges
+        w = rs.rand(n, 1) * 3 if weighted else 1.0     # the caller multiplies both by the sample weight
+        g = rs.randn(n, k) * w
+        h = np.maximum((rs.rand(n, k) + 0.05) * w, 1e-8)
+        fs = None
+        if frac < 1.0 and f > 1:
+            fs = rs.rand(f) < frac
+            fs[rs.randint(f)] = True
+        gr, cr = gu.both(X, g, h, levels=(n * depth <= 200000), max_depth=depth, split_samples=s, seed=seed,
+                         hist_cache_bytes=budget, feature_set=fs)
+        gu.assert_tree_parity(gr, cr, levels=(n * depth <= 200000))
+
+    run()
