@@ -250,6 +250,7 @@ struct TileWalk {
   int rpp;       // rows per pass of a workgroup (tile_rows / rows per lane)
   int n_gk;      // groups * outputs
   int n_chunks;  // row-tile ranges
+  bool all_resident;  // host side: the launch's workgroups all fit the chip at once
 };
 
 // Read-only inputs of the tile walk. They are separate __restrict__ kernel
@@ -1272,7 +1273,9 @@ int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& 
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
-    kRoot && a.w.n_gk > 1 && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr, sink);
+    // meeting points only between workgroups that run at the same time: one that waits for a
+    // workgroup not yet started would sit out its whole wait at every meeting point
+    kRoot && a.w.n_gk > 1 && a.w.all_resident && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr, sink);
   return LBT_OK;
 }
 template <typename BinT, int BV, bool kEmbed>
@@ -1300,6 +1303,7 @@ int fill_walk(TileWalk& w, const HistBatch& b, int n_cu, int n_groups, int rpp, 
   per_xcd         = std::min<int64_t>(per_xcd, std::max<int64_t>(1, (max_tiles + 7) / 8));
   w.n_chunks      = static_cast<int>(per_xcd * 8);
   *grid           = static_cast<unsigned>(per_xcd * 8 * w.n_gk);
+  w.all_resident  = static_cast<int64_t>(*grid) <= static_cast<int64_t>(per_cu) * n_cu;
   return LBT_OK;
 }
 
