@@ -1605,7 +1605,24 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     }
     budget -= 16 * 1024;
   }
-  // ... then the largest table, up to four cells per proposal, that still fits these groups
+  // ... half as many groups again where that buys a table of eight cells per proposal (wide
+  // inputs: with 125 features of 256 proposals in a group only two cells per proposal are left,
+  // and the search, no longer hidden behind the loads, sets the pace; a further group costs one
+  // more partly used cache line per row) ...
+  {
+    const int n_min   = static_cast<int>(sgroups.size()) - 1;
+    const int allowed = n_min + n_min / 2;
+    std::vector<int32_t> trial;
+    for (int c = kMaxCells; allowed > n_min && c >= 128; c >>= 1) {
+      if (c > 8 * std::max(16, max_feature_bins)) continue;
+      pack_groups(F, vec, vec, search_budget, [&](int f) { return search_bytes(f, c); }, trial);
+      if (widest_group(trial, [&](int f) { return search_bytes(f, c); }) > search_budget) continue;
+      if (static_cast<int>(trial.size()) - 1 > allowed) continue;
+      sgroups = trial;
+      break;
+    }
+  }
+  // ... then the largest table, up to eight cells per proposal, that still fits these groups
   int cells = 64;
   size_t search_lds = widest_group(sgroups, [&](int f) { return search_bytes(f, 64); });
   for (int c = 128; c <= kMaxCells && c <= 8 * std::max(16, max_feature_bins); c <<= 1) {
