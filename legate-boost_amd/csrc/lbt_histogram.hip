@@ -338,6 +338,13 @@ struct VecOf<double, 1> {
   using type = double;
 };
 
+// The same vectors for rows that start on a multiple of the element size only (a feature
+// count that is no multiple of the vector width): loaded with element alignment.
+template <typename T, int VEC>
+struct __attribute__((packed, aligned(sizeof(T)))) LooseVec {
+  T v[VEC];
+};
+
 // Number of proposals in [p, p+n) that are < x (branch-free, fixed trip count).
 template <typename T>
 __device__ inline int count_less(const T* p, int n, T x, int steps)
@@ -719,7 +726,11 @@ struct BinRowsArgs {
   const RecInfo* rec;         // [histogram groups]
 };
 
-template <typename T, int VEC, typename BinT>
+// kRagged: the feature count is no multiple of VEC. The last lane of a row then owns fewer
+// than VEC features: it loads the VEC values that end with the row's last one and takes its
+// own from their end, and its surplus bins are zeros in the record's padding. Rows then start
+// on element boundaries only, so all lanes load with element alignment.
+template <typename T, int VEC, typename BinT, bool kRagged>
 __global__ void __launch_bounds__(kHistThreads)
   bin_rows_kernel(BinRowsArgs<T> a, const T* __restrict__ X, const int2* __restrict__ qgh,
                   BinT* __restrict__ binned)
@@ -751,17 +762,20 @@ __global__ void __launch_bounds__(kHistThreads)
     const int words     = gs * (C / kCellsPerWord);
     for (int i = threadIdx.x; i < words; i += kHistThreads) s_cell[i] = src[i];
   }
-  // group widths are multiples of VEC, so every lane owns VEC real features
-  const int lanes_per_row = gs / VEC;
+  // group widths are multiples of VEC (but for the last group of a ragged feature count), so
+  // every lane owns VEC real features (the last lane of such a row: mine of them)
+  const int lanes_per_row = (gs + VEC - 1) / VEC;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
   const bool active       = rsub < a.rpp;
   const int fb            = f0 + lr * VEC;  // first feature of this lane
+  const int mine          = kRagged ? min(VEC, f1 - fb) : VEC;
+  const int shift         = VEC - mine;     // its values are the last `mine` of the VEC it loads
   T c_lo[VEC], c_invw[VEC];
   int c_cell[VEC], c_prop[VEC], c_end[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; v++) {
-    const int f = fb + v;
+    const int f = kRagged ? min(fb + v, f1 - 1) : fb + v;
     c_lo[v]   = a.cell_lo[f];
     c_invw[v] = a.cell_invw[f];
     c_cell[v] = (f - f0) * (C / kCellsPerWord);
@@ -775,20 +789,20 @@ __global__ void __launch_bounds__(kHistThreads)
   // with zero padding and, for single-output trees, the row's gradient pair in its last 8
   // bytes; where it can, the lane writes the record's last 16 bytes with one store, so that
   // every record reaches memory as whole, aligned pieces.
-  const int tg = a.bin_tail[fb + VEC - 1];
+  const int tg = a.bin_tail[fb + mine - 1];
   int tz_from = 0, tz_to = 0, tq = -1, t16 = 0;
   bool tz_words = false;
   int tmode     = 0;  // 1: zeros, then the pair on its own; 2: own bins + pair in one store; 3: zeros, then [0, 0, pair]
   if (tg > 0) {
     const RecInfo ri = a.rec[tg - 1];
     const int my_off = static_cast<int>(a.bin_base[fb] * static_cast<int64_t>(sizeof(BinT)) - ri.base);
-    tz_from          = ri.bins_end - my_off;
+    tz_from          = max(ri.bins_end - my_off, VEC * static_cast<int>(sizeof(BinT)));  // behind the lane's own store
     tz_to            = ri.zero_end - my_off;
     tq               = ri.q_off >= 0 ? ri.q_off - my_off : -1;
     tmode            = 1;
     if (VEC * sizeof(BinT) == 4 && ri.q_off >= 0 && ri.q_off == ri.size - 8) {
       t16 = ri.size - 16 - my_off;
-      if (t16 == 0 && ri.bins_end == my_off + 4) {
+      if (t16 == 0 && ri.bins_end <= my_off + 4) {
         tmode = 2;
       } else if (ri.bins_end <= ri.size - 16) {
         tmode = 3;
@@ -805,7 +819,7 @@ __global__ void __launch_bounds__(kHistThreads)
   // keeps a chunk's rows times the widest row below 2^31 bytes), which advance by a uniform
   // step from pass to pass instead of being multiplied out per row.
   const int n_local                  = static_cast<int>(r_end - r_begin);
-  const unsigned char* const x_chunk = reinterpret_cast<const unsigned char*>(X + r_begin * a.F + fb);
+  const unsigned char* const x_chunk = reinterpret_cast<const unsigned char*>(X + r_begin * a.F + fb - shift);
   const int2* const q_chunk          = qgh + r_begin;
   unsigned char* const b_chunk       = reinterpret_cast<unsigned char*>(bin_base + r_begin * pitch);
   const uint32_t row_bytes = static_cast<uint32_t>(a.F) * sizeof(T);
@@ -824,10 +838,17 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
       const uint32_t off = min(off0 + u * x_step, x_last);
-      if constexpr (VEC == 1)
+      if constexpr (VEC == 1) {
         xv[u] = *reinterpret_cast<const T*>(x_chunk + off);
-      else
+      } else if constexpr (kRagged) {
+        const LooseVec<T, VEC> lv = *reinterpret_cast<const LooseVec<T, VEC>*>(x_chunk + off);
+        if constexpr (VEC == 2)
+          xv[u] = Vec{lv.v[0], lv.v[1]};
+        else
+          xv[u] = Vec{lv.v[0], lv.v[1], lv.v[2], lv.v[3]};
+      } else {
         xv[u] = *reinterpret_cast<const Vec*>(x_chunk + off);
+      }
     }
   };
   auto search_pass = [&](int first, const Vec (&x_c)[kUnroll]) {
@@ -853,6 +874,20 @@ __global__ void __launch_bounds__(kHistThreads)
           xs[1] = x_c[u].y;
           xs[2] = x_c[u].z;
           xs[3] = x_c[u].w;
+        }
+        if constexpr (kRagged && VEC > 1) {
+          // the lane with fewer features took the values that end with the row's last one
+          T t[VEC];
+#pragma unroll
+          for (int v = 0; v < VEC; v++) t[v] = xs[v];
+#pragma unroll
+          for (int v = 0; v < VEC; v++) {
+            T x = t[v];
+#pragma unroll
+            for (int sh = 1; sh < VEC; sh++)
+              if (v + sh < VEC) x = shift == sh ? t[v + sh] : x;
+            xs[v] = x;
+          }
         }
         BinT rel[VEC];
         // the table gives a proposal at or before the value's bin; the proposals from there on
@@ -881,6 +916,7 @@ __global__ void __launch_bounds__(kHistThreads)
             }
           }
           rel[v] = static_cast<BinT>(bn[v] + cnt[v] - c_prop[v]);
+          if constexpr (kRagged) rel[v] = v < mine ? rel[v] : BinT(0);
         }
         unsigned char* tail = b_chunk + (b_off0 + u * b_step);
         BinT* bp            = reinterpret_cast<BinT*>(tail);
@@ -1247,21 +1283,27 @@ int launch_search_rows(hipStream_t stream, const HistSetup& hs, const HistArgs<T
   return launch_search<T, VEC, false>(stream, hs, a, b, grid);
 }
 
-template <typename T, int VEC, typename BinT>
+template <typename T, int VEC, typename BinT, bool kRagged>
 int launch_bin_rows(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
 {
   static bool attr_set[kMaxDevices] = {};
-  LBT_TRY(allow_dynamic_lds(bin_rows_kernel<T, VEC, BinT>, kLdsBudget, attr_set));
-  bin_rows_kernel<T, VEC, BinT><<<grid, kHistThreads, hs.lds_bytes, stream>>>(a, static_cast<const T*>(b.X), b.qgh,
-                                                                            static_cast<BinT*>(hs.binned));
+  LBT_TRY(allow_dynamic_lds(bin_rows_kernel<T, VEC, BinT, kRagged>, kLdsBudget, attr_set));
+  bin_rows_kernel<T, VEC, BinT, kRagged><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
+    a, static_cast<const T*>(b.X), b.qgh, static_cast<BinT*>(hs.binned));
   return LBT_OK;
 }
 
 template <typename T, int VEC>
 int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
 {
-  if (hs.bin_bytes == 1) return launch_bin_rows<T, VEC, uint8_t>(stream, hs, a, b, grid);
-  return launch_bin_rows<T, VEC, uint16_t>(stream, hs, a, b, grid);
+  if constexpr (VEC > 1) {
+    if (hs.ragged) {
+      if (hs.bin_bytes == 1) return launch_bin_rows<T, VEC, uint8_t, true>(stream, hs, a, b, grid);
+      return launch_bin_rows<T, VEC, uint16_t, true>(stream, hs, a, b, grid);
+    }
+  }
+  if (hs.bin_bytes == 1) return launch_bin_rows<T, VEC, uint8_t, false>(stream, hs, a, b, grid);
+  return launch_bin_rows<T, VEC, uint16_t, false>(stream, hs, a, b, grid);
 }
 
 template <typename BinT, int BV, bool kEmbed, bool kRoot>
@@ -1566,6 +1608,17 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   // widest aligned vector of features a lane can load from X
   int vec = is_f64 ? 2 : 4;
   while (vec > 1 && (F % vec != 0 || reinterpret_cast<uintptr_t>(X) % 16 != 0)) vec >>= 1;
+  // The binning pass keeps the full width for a feature count that is no multiple of it (the
+  // last lane of a row then owns fewer features); the kernel that searches X itself does not.
+  hs.ragged = false;
+  if (hs.binned != nullptr) {
+    const int full = is_f64 ? 2 : 4;
+    if (vec < full && F >= full && reinterpret_cast<uintptr_t>(X) % elem == 0) {
+      vec       = full;
+      hs.ragged = F % full != 0;
+      if (!hs.ragged && reinterpret_cast<uintptr_t>(X) % 16 != 0) hs.ragged = true;  // same loads: element alignment
+    }
+  }
   hs.vec = vec;
   int max_feature_bins = 1;
   for (int f = 0; f < F; f++) max_feature_bins = std::max(max_feature_bins, rp[f + 1] - rp[f]);

@@ -341,6 +341,7 @@ struct HistSetup {
   void* binned         = nullptr;  // null: cache off
   size_t binned_capacity = 0;      // bytes available at `binned`
   int bin_bytes        = 0;        // 1 or 2
+  bool ragged          = false;    // binning pass: rows are no whole number of lane vectors (or start unaligned)
   int bvec             = 1;        // cached bins a lane of the histogram kernel loads at once
   bool embed           = false;    // records carry the row's (grad, hess)
   size_t blds_bytes    = 0;        // LDS of the histogram kernel (packed sub-histogram only)

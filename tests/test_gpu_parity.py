@@ -32,6 +32,11 @@ def _problem(seed, n, f, k, dtype=np.float32, lowcard=True):
     (4000, 150, 1, 4, 256, np.float32),   # several feature groups, two features per lane
     (6000, 64, 1, 5, 256, np.float32),    # one group, gradients embedded in the bin records
     (2500, 18, 1, 4, 300, np.float64),    # two-byte bins with double features
+    (4000, 5, 1, 4, 64, np.float32),      # feature counts that are no multiple of a lane's four: the
+    (4000, 6, 1, 4, 64, np.float32),      # last lane of a row owns 1, 2 or 3 features
+    (4000, 103, 2, 4, 256, np.float32),
+    (3000, 9, 1, 4, 64, np.float64),      # ... or of a lane's two doubles
+    (3000, 11, 1, 3, 400, np.float32),    # ... with two-byte bins
 ])
 def test_build_tree_bit_exact(n, f, k, depth, s, dtype):
     import gpu_util as gu
@@ -482,3 +487,23 @@ def test_property_sweep_against_the_oracle():
         gu.assert_tree_parity(gr, cr, levels=(n * depth <= 200000))
 
     run()
+
+
+@pytest.mark.parametrize("f,dtype,skip", [(8, np.float32, 1), (6, np.float32, 3), (7, np.float32, 2), (5, np.float64, 1)])
+def test_matrix_that_starts_off_a_16_byte_boundary(f, dtype, skip):
+    """X as a view that begins `skip` elements into an allocation: rows then start on element
+    boundaries only, which the binning pass has to load as such."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    n = 3000
+    X, g, h = _problem(f + skip, n, f, 1, dtype)
+    base = torch.zeros(n * f + skip, dtype=torch.from_numpy(X).dtype, device="cuda")
+    Xd = base[skip:].view(n, f)
+    Xd.copy_(torch.from_numpy(X))
+    assert Xd.data_ptr() % 16 != 0 and Xd.is_contiguous()
+    gr = ops.build_tree(Xd, torch.from_numpy(g).cuda(), torch.from_numpy(h).cuda(), max_depth=5, split_samples=64,
+                        seed=31, taps=True, row_leaf=True)
+    cr = orc.build_tree(X, g, h, max_depth=5, split_samples=64, seed=31)
+    gu.assert_tree_parity(gr, cr)
