@@ -203,7 +203,7 @@ typedef struct lbt_packed_ensemble {
   int32_t n_batches; /* groups of trees that are staged in the LDS together */
   int32_t lanes;     /* lanes that share a row in the traversal kernel (4, 8 or 16; set by n_features) */
   int32_t lds_bytes; /* LDS of one workgroup: its row tile and the widest batch of nodes */
-  int32_t reserved;
+  int32_t few_trees; /* 1: at most `lanes` trees, walked one per lane */
   int64_t total_nodes;
 } lbt_packed_ensemble;
 

@@ -141,16 +141,19 @@ constexpr int kPackBatches  = 128; // batch descriptors written per launch
 constexpr int kTileThreads  = 1024;
 // L lanes share a row; a workgroup then covers 1024 / L rows, and a batch holds L * kLaneTrees
 // trees. Wide feature matrices take more lanes per row, so that the row tile still fits the LDS.
-template <int L>
+// kFew: an ensemble of at most L trees (the one tree a boosting round predicts with): one tree
+// per lane, so that no lane walks a tree that is not there.
+template <int L, bool kFew = false>
 struct TileShape {
   static constexpr int kRowLanes   = L;
   static constexpr int kRows       = kTileThreads / L;
-  static constexpr int kLaneTrees  = L == 4 ? 5 : (L == 8 ? 3 : 2);
+  static constexpr int kLaneTrees  = kFew ? 1 : (L == 4 ? 5 : (L == 8 ? 3 : 2));
   static constexpr int kBatchTrees = kRowLanes * kLaneTrees;
 };
 constexpr int kTileMaxK     = 8;
 constexpr size_t kTileLds   = 160 * 1024 - 2048;  // dynamic LDS of the tile kernel
 constexpr int kCopyWords    = 6;  // 16-byte words a thread moves per batch: 6 * 1024 * 16 B >= any batch
+constexpr size_t kSmallEnsembleLds = 78 * 1024;  // row tile + nodes of a small ensemble: two workgroups per CU
 constexpr int kMaxPackedNodes = 65535;  // the right child of a float node has 16 bits
 
 struct PackBatch {
@@ -266,7 +269,9 @@ __device__ __forceinline__ Prefetched<S> fetch_batch(const BatchInfo& bi, const 
 #pragma unroll
   for (int c = 0; c < kCopyWords; c++) {
     const int i = threadIdx.x + c * kTileThreads;
-    pf.words[c] = src[i < n16 ? i : 0];
+    // one tree per lane: words past the batch are not asked for (a single tree is a quarter of
+    // one round of the threads); full batches load all of them without a test
+    if (S::kLaneTrees > 1 || c * kTileThreads < n16) pf.words[c] = src[i < n16 ? i : 0];
   }
 #pragma unroll
   for (int j = 0; j < S::kLaneTrees; j++) {
@@ -312,14 +317,14 @@ __device__ __forceinline__ void add_leaves_in_order(double (&acc)[kAcc], const i
   add_leaves_from<S, kAcc, 0>(acc, at, cnt, batch_leaves, K);
 }
 
-template <typename T, bool kSingle, int L>
+template <typename T, bool kSingle, int L, bool kFew = false>
 __global__ void __launch_bounds__(kTileThreads)
   predict_tile_kernel(const T* __restrict__ X, int64_t n_rows, int F, int pitch, int n_batches,
                       const BatchInfo* __restrict__ batches, const PackedTree* __restrict__ desc,
                       const PackedNode<T>* __restrict__ nodes, const double* __restrict__ leaves, int K,
                       double* __restrict__ out)
 {
-  using S = TileShape<L>;
+  using S = TileShape<L, kFew>;
   constexpr int kTileRows = S::kRows, kLaneTrees = S::kLaneTrees;
   extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
   T* s_x = reinterpret_cast<T*>(smem_raw);
@@ -498,15 +503,17 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
   if (all_nodes <= 24 * 1024) {
     for (int l : {4, 8, 16}) {
       const size_t xb = (static_cast<size_t>(kTileThreads / l) * (F | 1) * sizeof(T) + 15) & ~size_t(15);
-      if (l >= lanes && xb + all_nodes <= 78 * 1024) {
+      if (l >= lanes && xb + all_nodes <= kSmallEnsembleLds) {
         lanes   = l;
         x_bytes = xb;
         break;
       }
     }
   }
-  const int batch_trees = lanes == 4 ? TileShape<4>::kBatchTrees
-                                     : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees);
+  const bool few        = n_trees <= lanes;
+  const int batch_trees = few ? lanes
+                              : (lanes == 4 ? TileShape<4>::kBatchTrees
+                                            : (lanes == 8 ? TileShape<8>::kBatchTrees : TileShape<16>::kBatchTrees));
   constexpr int kNodesPerWord = 16 / sizeof(PackedNode<T>);
   const int64_t node_cap = std::min<int64_t>(static_cast<int64_t>((kTileLds - x_bytes) / sizeof(PackedNode<T>)),
                                              static_cast<int64_t>(kCopyWords) * kTileThreads * kNodesPerWord);
@@ -576,6 +583,7 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
   ens->n_trees     = n_trees;
   ens->n_batches   = n_batches;
   ens->lanes       = lanes;
+  ens->few_trees   = few ? 1 : 0;
   // the row tile and the widest batch of nodes (whole 16-byte words)
   ens->lds_bytes   = static_cast<int32_t>(
     x_bytes + ((static_cast<size_t>(widest_batch + kNodesPerWord) * sizeof(PackedNode<T>) + 15) & ~size_t(15)));
@@ -600,8 +608,19 @@ int run_tiled(hipStream_t stream, const T* X, int64_t N, const lbt_packed_ensemb
     return LBT_OK;
   };
   static bool attr[6][kMaxDevices] = {};
+  static bool attr_few[6][kMaxDevices] = {};
   const bool single = K == 1;
-  if (lanes == 4)
+  if (ens.few_trees == 1) {
+    if (lanes == 4)
+      LBT_TRY(single ? launch(predict_tile_kernel<T, true, 4, true>, attr_few[0])
+                     : launch(predict_tile_kernel<T, false, 4, true>, attr_few[1]));
+    else if (lanes == 8)
+      LBT_TRY(single ? launch(predict_tile_kernel<T, true, 8, true>, attr_few[2])
+                     : launch(predict_tile_kernel<T, false, 8, true>, attr_few[3]));
+    else
+      LBT_TRY(single ? launch(predict_tile_kernel<T, true, 16, true>, attr_few[4])
+                     : launch(predict_tile_kernel<T, false, 16, true>, attr_few[5]));
+  } else if (lanes == 4)
     LBT_TRY(single ? launch(predict_tile_kernel<T, true, 4>, attr[0]) : launch(predict_tile_kernel<T, false, 4>, attr[1]));
   else if (lanes == 8)
     LBT_TRY(single ? launch(predict_tile_kernel<T, true, 8>, attr[2]) : launch(predict_tile_kernel<T, false, 8>, attr[3]));

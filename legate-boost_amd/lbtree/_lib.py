@@ -79,7 +79,7 @@ class PackedEnsemble(C.Structure):
         ("n_batches", C.c_int32),
         ("lanes", C.c_int32),
         ("lds_bytes", C.c_int32),
-        ("reserved", C.c_int32),
+        ("few_trees", C.c_int32),
         ("total_nodes", C.c_int64),
     ]
 
