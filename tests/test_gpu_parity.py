@@ -507,3 +507,30 @@ def test_matrix_that_starts_off_a_16_byte_boundary(f, dtype, skip):
                         seed=31, taps=True, row_leaf=True)
     cr = orc.build_tree(X, g, h, max_depth=5, split_samples=64, seed=31)
     gu.assert_tree_parity(gr, cr)
+
+
+@pytest.mark.parametrize("f,lanes", [(13, 4), (100, 8), (330, 16)])
+@pytest.mark.parametrize("k", [1, 3])
+def test_predict_with_a_handful_of_trees(f, lanes, k):
+    """Ensembles of at most as many trees as lanes share a row are walked one tree per lane: a
+    single tree (what a boosting round predicts with), exactly that many, and one more (the
+    general shape again)."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(f * 7 + k)
+    X = rs.rand(5003, f).astype(np.float32)
+    trees_c, trees_g = [], []
+    for t in range(lanes + 1):
+        depth = [6, 2, 8, 4][t % 4]
+        m, inner = 2 ** (depth + 1) - 1, 2 ** depth - 1
+        feat = -np.ones(m, np.int32)
+        feat[:inner] = rs.randint(0, f, inner)
+        split = rs.rand(m)
+        leaf = rs.randn(m, k)
+        trees_c.append((leaf, feat, split))
+        trees_g.append(tuple(ops.as_device(a) for a in (leaf, feat, split)))
+    for n_trees in (1, 2, lanes, lanes + 1):
+        want = orc.predict(X, trees_c[:n_trees], k)
+        assert np.array_equal(gu.cpu(ops.predict(X, trees_g[:n_trees], k)), want), n_trees
