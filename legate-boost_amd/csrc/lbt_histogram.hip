@@ -1478,8 +1478,10 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
 // Packs consecutive features, `unit` at a time, into groups whose LDS need
 // (bytes_of(feature)) stays within the budget and whose rows take at most half a
 // workgroup of lanes (lane_vec features per lane); a second pass balances widths.
+// more_groups: that many groups beyond the fewest the budget allows.
 template <typename BytesOf>
-size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_of, std::vector<int32_t>& groups)
+size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_of, std::vector<int32_t>& groups,
+                   int more_groups = 0)
 {
   const int max_lanes = kHistThreads / 2;  // at least two rows per pass
   size_t lds          = 0;
@@ -1504,7 +1506,7 @@ size_t pack_groups(int F, int unit, int lane_vec, size_t budget, BytesOf bytes_o
     lds = std::max(lds, cur);
   };
   pack(F + unit);  // fewest groups the LDS allows
-  const int n_min = static_cast<int>(groups.size()) - 1;
+  const int n_min = std::min(static_cast<int>(groups.size()) - 1 + more_groups, (F + unit - 1) / unit);
   int target      = (F + n_min - 1) / n_min;
   target          = ((target + unit - 1) / unit) * unit;
   pack(target);    // same count where the budget allows, balanced widths
@@ -1704,6 +1706,28 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     // histogram groups hold whole lanes of the binning pass (multiples of vec features)
     const size_t hbudget = kLdsBudget - 8 * kHistThreads;  // one spare slot per lane
     pack_groups(F, vec, hs.bvec, hbudget, hist_bytes, groups);
+    {
+      // A launch has one workgroup per (row range, group, output) and as many row ranges as keep
+      // every CU busy once: 3 groups x 8 outputs are 24 workgroups per row range, of which a
+      // 32-CU XCD takes one set and leaves 8 CUs idle. One or two groups more are taken when that
+      // fills the chip a quarter better (the atomics per row stay the same, the record requests
+      // per row grow with the groups).
+      int device = 0, n_cu = 256;
+      LBT_HIP(hipGetDevice(&device));
+      LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
+      const int slots = std::max(1, n_cu / 8);  // workgroups of this size that an XCD runs at once
+      auto filled = [&](int n_groups) {
+        const int n_gk = n_groups * K;
+        if (n_gk <= slots) return static_cast<double>(slots / n_gk * n_gk) / slots;
+        const int rounds = (n_gk + slots - 1) / slots;
+        return static_cast<double>(n_gk) / (static_cast<double>(rounds) * slots);
+      };
+      const int n0 = static_cast<int>(groups.size()) - 1;
+      int best     = 0;
+      for (int more = 1; more <= 2; more++)
+        if (filled(n0 + more) >= 1.25 * filled(n0) && filled(n0 + more) > filled(n0 + best)) best = more;
+      if (best > 0) pack_groups(F, vec, hs.bvec, hbudget, hist_bytes, groups, best);
+    }
     const size_t blds = widest_group(groups, hist_bytes);
     if (blds > hbudget) {
       set_error("the bins of one feature group do not fit the LDS (%zu bytes)", blds);
