@@ -379,7 +379,8 @@ inline int64_t bin_row_bytes_max(int n_features, int split_samples)
   int64_t cap = static_cast<int64_t>((kLdsBudget - 8 * kHistThreads) / (8 * static_cast<size_t>(split_samples)));
   if (cap >= 4) cap = cap / 4 * 4;
   if (cap < 1) cap = 1;
-  const int64_t groups_max = (n_features + cap - 1) / cap + 1;
+  // one more for the uneven widths of a balanced split, two more that may be taken to fill idle CUs
+  const int64_t groups_max = (n_features + cap - 1) / cap + 3;
   return static_cast<int64_t>(n_features) * bin_bytes + groups_max * 48;
 }
 

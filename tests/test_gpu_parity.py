@@ -37,6 +37,8 @@ def _problem(seed, n, f, k, dtype=np.float32, lowcard=True):
     (4000, 103, 2, 4, 256, np.float32),
     (3000, 9, 1, 4, 64, np.float64),      # ... or of a lane's two doubles
     (3000, 11, 1, 3, 400, np.float32),    # ... with two-byte bins
+    (2000, 200, 8, 3, 256, np.float32),   # 3 groups x 8 outputs would leave CUs idle: a fourth group is taken
+    (2000, 300, 5, 3, 256, np.float32),
 ])
 def test_build_tree_bit_exact(n, f, k, depth, s, dtype):
     import gpu_util as gu
