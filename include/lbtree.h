@@ -40,6 +40,18 @@ extern "C" {
 const char* lbt_last_error(void);
 int lbt_version(void);
 
+/*
+ * State the library keeps between calls, all of it per host thread: the error string, and, once
+ * the thread has called lbt_build_tree, two small pinned host buffers and three events (the
+ * values a build reads back while it runs, and the staging buffer of the tables it sends).
+ * They are created on first use and reused; this call waits for the copies that still use them
+ * and frees them (the next build on the thread creates them again). A thread that ends without
+ * calling it leaves them allocated until the process ends. Beyond these and the optional
+ * profiler there is no global state; no device pointer is kept after a call returns.
+ * No counterpart in the reference (Legate owns its task-scoped buffers).
+ */
+int lbt_release_thread_resources(void);
+
 /* The eight task scalars of BUILD_TREE in their reference order
  * (legateboost/models/tree.py:121-129, build_tree.cu:1292-1299), plus the
  * histogram-cache budget that the reference hard-codes to 1e9 bytes
@@ -100,7 +112,15 @@ size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_
  *             [max_nodes] f64, [max_nodes][n_outputs] f64)
  *   workspace    device scratch of at least lbt_build_tree_workspace_bytes(...)
  * The call returns after the stream has been synchronised, like the
- * reference (build_tree.cu:1356).
+ * reference (build_tree.cu:1356), also when it returns an error: no kernel of a
+ * failed call is still queued, so outputs and workspace may be released at once.
+ *
+ * Gradients and hessians of either sign are rounded and summed exactly as the
+ * reference does in int64 (build_tree.cu:112-129). One case is refused with
+ * LBT_ERR_UNSUPPORTED instead: a rounded value of magnitude 2^31, which needs a
+ * single entry that holds the entire absolute sum of g (or of h) and a stochastic
+ * rounding that takes it upwards. Every other value fits the signed 32 bits the
+ * kernels store (|v| * (2^31 - 1) / sum|v| <= 2^31 - 1).
  */
 int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
                    int64_t n_rows, int32_t n_features, const double* g, const double* h,
@@ -116,8 +136,11 @@ int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_off
  * lbt_build_tree on the same workspace) needs; the reference synchronises (build_tree.cu:1356)
  * although Legate orders tasks on the task stream. The members of `taps` that hold host
  * values read back from the device (scales, level_instances, level_built_instances,
- * level_built_nodes) are not filled. Errors of kernels surface at the caller's next
- * synchronisation.
+ * level_built_nodes) are not filled. A status other than LBT_OK (invalid arguments, or the
+ * 2^31 case above, which is noticed when the first level has been queued) is returned like in
+ * the synchronising form, but kernels queued before the failure may still be running: the
+ * caller synchronises the stream before it releases outputs or workspace. Faults inside
+ * kernels surface at the caller's next synchronisation.
  */
 int lbt_build_tree_async(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
                          int64_t n_rows, int32_t n_features, const double* g, const double* h,
@@ -153,8 +176,8 @@ int lbt_select_split_samples(void* stream, const void* X, int32_t x_dtype, int64
  *   root_sums  device int64 [n_outputs][2]
  *   scales     device double [4]: scale.grad, scale.hess, 1/scale.grad, 1/scale.hess
  *   workspace  device scratch of lbt_quantise_gradients_workspace_bytes(...)
- * Enqueues on the stream, does not wait. A rounded value that does not fit 32 bits is
- * stored truncated here; lbt_build_tree reports it as LBT_ERR_UNSUPPORTED.
+ * Enqueues on the stream, does not wait. A rounded value of magnitude 2^31 (see
+ * lbt_build_tree) is stored truncated here; lbt_build_tree reports it as LBT_ERR_UNSUPPORTED.
  */
 size_t lbt_quantise_gradients_workspace_bytes(int64_t n_rows, int32_t n_outputs);
 int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64_t n_rows, int32_t n_outputs,

@@ -242,8 +242,9 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
-// qstats[0] = max over all entries of max(|q.grad|, q.hess); qstats[1] != 0 if a
-// value does not fit the packed int32 form.
+// qstats[0] = max over all entries of max(|q.grad|, |q.hess|); qstats[1] != 0 if a
+// value does not fit the packed int32 form (|q| = 2^31: a single entry that holds the whole
+// absolute sum, rounded up).
 __global__ void scales_kernel(const double* sum_a, const double* sum_b, double* scales,
                               unsigned long long* qstats)
 {
@@ -289,7 +290,7 @@ __global__ void __launch_bounds__(kThreads)
     int64_t qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
     x = minstd_next(x);
     int64_t qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
-    bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
+    bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < -2147483647LL;
     q_out[row * K + k] = make_int2(static_cast<int>(qg), static_cast<int>(qh));
     unsigned long long ag = static_cast<unsigned long long>(qg < 0 ? -qg : qg);
     unsigned long long ah = static_cast<unsigned long long>(qh < 0 ? -qh : qh);
@@ -361,7 +362,7 @@ __global__ void __launch_bounds__(kThreads)
       int64_t qg = static_cast<int64_t>(floor(scaled_grad) + static_cast<double>(uniform01(x) < grad_remainder));
       x = minstd_next(x);
       int64_t qh = static_cast<int64_t>(floor(scaled_hess) + static_cast<double>(uniform01(x) < hess_remainder));
-      bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < 0;
+      bad |= qg > 2147483647LL || qg < -2147483647LL || qh > 2147483647LL || qh < -2147483647LL;
       q_out[e] = make_int2(static_cast<int>(qg), static_cast<int>(qh));
       unsigned long long ag = static_cast<unsigned long long>(qg < 0 ? -qg : qg);
       unsigned long long ah = static_cast<unsigned long long>(qh < 0 ? -qh : qh);
@@ -1152,6 +1153,8 @@ struct Layout {
   double* proposals_d;
   int32_t* row_pointers;
   int32_t* bin_feature;
+  void* upload_block;
+  size_t upload_bytes;
   int32_t* groups;
   int32_t* sgroups;
   int64_t* bin_base;
@@ -1220,12 +1223,16 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.proposals_d  = ar.take<double>(static_cast<size_t>(F) * S);
   L.row_pointers = ar.take<int32_t>(F + 1);
   L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
+  // the tables hist_prepare sends from the host: one block, filled by one copy
+  const size_t upload_at = ar.used;
   L.groups       = ar.take<int32_t>(F + 1);
   L.sgroups      = ar.take<int32_t>(F + 1);
   L.bin_base     = ar.take<int64_t>(F);
   L.bin_stride   = ar.take<int32_t>(F);
   L.bin_tail     = ar.take<int32_t>(F);
   L.rec          = ar.take<RecInfo>(F);
+  L.upload_block = L.groups;
+  L.upload_bytes = ar.used - upload_at;
   // bin cache: one or two bytes per (row, feature); used when the tree has at least two levels
   L.binned_bytes = max_depth >= 2 ? static_cast<size_t>(N) * bin_row_bytes_max(F, S) : 0;
   L.binned       = max_depth >= 2 ? static_cast<void*>(ar.take<char>(L.binned_bytes + 16)) : nullptr;
@@ -1296,24 +1303,21 @@ int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
 // What the host reads back in the middle of a call (bin counts per feature, the quantiser's
 // overflow flag): pinned memory and two events per host thread, so that each value is waited
 // for by itself and not together with everything else that is queued on the stream.
-struct HostMirror {
-  int32_t* pinned = nullptr;  // [4 + capacity]: two 64-bit quantiser statistics, then the row pointers
-  size_t capacity = 0;
-  hipEvent_t counts_here = nullptr, stats_here = nullptr;
-};
-
-int host_mirror(int F, HostMirror** out)
+int host_mirror(int F, ThreadResources** out)
 {
-  static thread_local HostMirror hm;
+  ThreadResources& hm = thread_resources();
   if (hm.counts_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.counts_here, hipEventDisableTiming));
   if (hm.stats_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.stats_here, hipEventDisableTiming));
+  // an earlier call of this thread that did not wait (or failed half-way) may still own the buffer
+  LBT_HIP(hipEventSynchronize(hm.counts_here));
+  LBT_HIP(hipEventSynchronize(hm.stats_here));
   const size_t need = static_cast<size_t>(F) + 1;
-  if (hm.capacity < need) {
-    if (hm.pinned != nullptr) LBT_HIP(hipHostFree(hm.pinned));
-    hm.pinned   = nullptr;
-    hm.capacity = 0;
-    LBT_HIP(hipHostMalloc(reinterpret_cast<void**>(&hm.pinned), sizeof(int32_t) * (4 + need), hipHostMallocDefault));
-    hm.capacity = need;
+  if (hm.mirror_capacity < need) {
+    if (hm.mirror != nullptr) LBT_HIP(hipHostFree(hm.mirror));
+    hm.mirror          = nullptr;
+    hm.mirror_capacity = 0;
+    LBT_HIP(hipHostMalloc(reinterpret_cast<void**>(&hm.mirror), sizeof(int32_t) * (4 + need), hipHostMallocDefault));
+    hm.mirror_capacity = need;
   }
   *out = &hm;
   return LBT_OK;
@@ -1391,9 +1395,9 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   }
 
   // ---- split proposals
-  HostMirror* hm = nullptr;
+  ThreadResources* hm = nullptr;
   LBT_TRY(host_mirror(F, &hm));
-  int32_t* const rp_here = hm->pinned + 4;
+  int32_t* const rp_here = hm->mirror + 4;
   {
     ProfScope ps(LBT_PROF_PROPOSALS, stream);
     LBT_TRY(run_split_samples<T>(stream, X, row_offset, N, F, S, prm.seed, prm.dataset_rows, static_cast<T*>(L.draft),
@@ -1410,8 +1414,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization);
   }
-  const unsigned long long* const h_qstats = reinterpret_cast<const unsigned long long*>(hm->pinned);
-  LBT_HIP(hipMemcpyAsync(hm->pinned, L.qstats, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, stream));
+  const unsigned long long* const h_qstats = reinterpret_cast<const unsigned long long*>(hm->mirror);
+  LBT_HIP(hipMemcpyAsync(hm->mirror, L.qstats, 2 * sizeof(unsigned long long), hipMemcpyDeviceToHost, stream));
   LBT_HIP(hipEventRecord(hm->stats_here, stream));
   bool stats_checked = false;
   // a gradient that does not fit 32 bits ends the call; asked once a level's work is queued,
@@ -1421,7 +1425,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     stats_checked = true;
     LBT_HIP(hipEventSynchronize(hm->stats_here));
     if (h_qstats[1] != 0) {
-      set_error("a quantised gradient does not fit 32 bits: the gradient mass sits in a single entry");
+      set_error("a quantised gradient or hessian reaches 2^31 and does not fit the packed 32-bit form: one entry "
+                "holds the whole absolute sum and was rounded up");
       return LBT_ERR_UNSUPPORTED;
     }
     return LBT_OK;
@@ -1456,6 +1461,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   hs.bin_stride = L.bin_stride;
   hs.bin_tail   = L.bin_tail;
   hs.rec        = L.rec;
+  hs.upload_block = L.upload_block;
+  hs.upload_bytes = L.upload_bytes;
   // feature-major bins for the position updates of levels 0 .. max_depth-2 (and the final leaves)
   hs.bins_t        = L.binned != nullptr ? L.bins_t : nullptr;
   hs.bins_t_stride = L.bins_t_stride;
@@ -1782,9 +1789,13 @@ static int build_tree_entry(void* stream, const void* X, int32_t x_dtype, int64_
   else
     rc = lbt::build_tree_impl<double>(s, static_cast<const double*>(X), row_offset, n_rows, n_features, g, h, n_outputs,
                                       feature_set, *params, leaf, feature, split, gain, hessian, L, taps, sync_at_end);
-  if (rc != LBT_OK && lbt::profiler().mode != 0) {
-    (void)hipStreamSynchronize(s);
-    lbt::profiler().collect();
+  if (rc != LBT_OK) {
+    // Kernels of the stages before the failure may still be queued and write to the outputs and
+    // the workspace. The synchronising entry drains them, so that the caller may release both as
+    // soon as it sees the status (the task glue throws, and Legate then frees the buffers); the
+    // message of the failure is kept. The asynchronous entry leaves the wait to its caller.
+    if (sync_at_end || lbt::profiler().mode != 0) (void)hipStreamSynchronize(s);
+    if (lbt::profiler().mode != 0) lbt::profiler().collect();
   }
   return rc;
 }

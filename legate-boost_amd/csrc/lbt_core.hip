@@ -15,6 +15,12 @@ void set_error(const char* fmt, ...)
   va_end(ap);
 }
 
+ThreadResources& thread_resources()
+{
+  static thread_local ThreadResources tr;
+  return tr;
+}
+
 Profiler& profiler()
 {
   static Profiler p;
@@ -122,7 +128,23 @@ extern "C" {
 
 const char* lbt_last_error(void) { return lbt::g_error; }
 
-int lbt_version(void) { return 1; }
+int lbt_version(void) { return 2; }
+
+int lbt_release_thread_resources(void)
+{
+  lbt::ThreadResources& tr = lbt::thread_resources();
+  // the buffers may still feed or receive copies of calls that did not wait
+  if (tr.stage_free != nullptr) LBT_HIP(hipEventSynchronize(tr.stage_free));
+  if (tr.counts_here != nullptr) LBT_HIP(hipEventSynchronize(tr.counts_here));
+  if (tr.stats_here != nullptr) LBT_HIP(hipEventSynchronize(tr.stats_here));
+  if (tr.stage != nullptr) LBT_HIP(hipHostFree(tr.stage));
+  if (tr.mirror != nullptr) LBT_HIP(hipHostFree(tr.mirror));
+  if (tr.stage_free != nullptr) LBT_HIP(hipEventDestroy(tr.stage_free));
+  if (tr.counts_here != nullptr) LBT_HIP(hipEventDestroy(tr.counts_here));
+  if (tr.stats_here != nullptr) LBT_HIP(hipEventDestroy(tr.stats_here));
+  tr = lbt::ThreadResources{};
+  return LBT_OK;
+}
 
 void lbt_profile_enable(int on) { lbt::profiler().mode = on < 0 ? 0 : on; }
 

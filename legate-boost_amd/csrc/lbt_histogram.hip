@@ -18,10 +18,10 @@
 //     10M x 100 matrix with 256 proposals each are one group).
 //   * The packed sub-histogram of a histogram group of features (8 bytes per bin)
 //     is the only LDS state of the histogram kernel. (grad, hess) of a row are
-//     one 64-bit word (grad in the high half, hess unsigned in the low half)
+//     one 64-bit word (grad * 2^32 + hess, both signed; see pack_pair)
 //     added with a single LDS atomic; the sub-histogram is merged into the int64
 //     histogram with global atomics when the workgroup moves to another node.
-//     Before the low half or the signed high half could overflow
+//     Before either half could overflow
 //     (rows * max |q| >= 2^31) it is merged early; rows of tiny nodes go
 //     straight to global atomics.
 //   * The cache is stored histogram group by histogram group, [group][row][record].
@@ -360,6 +360,22 @@ __device__ inline int count_less(const T* p, int n, T x, int steps)
 }
 
 
+// A (grad, hess) pair as one 64-bit addend: grad * 2^32 + hess, both signed. Sums of such
+// words are sums of both halves as long as each total stays inside (-2^31, 2^31): the low
+// 32 bits of the sum, read as a signed number, are the hess total, and what is left after
+// taking it away is the grad total times 2^32. A negative hess (custom objectives) borrows
+// from the high half when it is packed and gives the borrow back when it is unpacked.
+__device__ __forceinline__ unsigned long long pack_pair(int grad, int hess)
+{
+  return (static_cast<unsigned long long>(static_cast<uint32_t>(grad + (hess >> 31))) << 32) |
+         static_cast<unsigned long long>(static_cast<uint32_t>(hess));
+}
+__device__ __forceinline__ void unpack_pair(unsigned long long v, int32_t& grad, int32_t& hess)
+{
+  hess = static_cast<int32_t>(static_cast<uint32_t>(v));
+  grad = static_cast<int32_t>(static_cast<uint32_t>(v >> 32)) - (hess >> 31);
+}
+
 // Merge of the packed LDS sub-histogram into the int64 histogram of a node.
 __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst)
 {
@@ -370,8 +386,8 @@ __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I
     const int i          = t + start < nb ? t + start : t + start - nb;
     unsigned long long v = s_hist[i];
     if (v != 0) {
-      int32_t gv  = static_cast<int32_t>(v >> 32);
-      uint32_t hv = static_cast<uint32_t>(v);
+      int32_t gv, hv;
+      unpack_pair(v, gv, hv);
       if (gv != 0) atomic_add_i64(&dst[i].grad, static_cast<int64_t>(gv));
       if (hv != 0) atomic_add_i64(&dst[i].hess, static_cast<int64_t>(hv));
       s_hist[i] = 0;
@@ -402,9 +418,11 @@ __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I6
     for (int i = threadIdx.x; i < nb; i += kHistThreads) {
       const unsigned long long v = s_hist[i];
       if (v != 0) {
+        int32_t gv, hv;
+        unpack_pair(v, gv, hv);
         I64Pair p = dst[i];
-        p.grad += static_cast<int32_t>(v >> 32);
-        p.hess += static_cast<uint32_t>(v);
+        p.grad += gv;
+        p.hess += hv;
         dst[i]    = p;
         s_hist[i] = 0;
       }
@@ -471,14 +489,17 @@ __global__ void __launch_bounds__(kHistThreads)
     for (int u = 0; u < 8; u++) v[u] = src[static_cast<int64_t>(list[i + u * step]) * sink.stride];
 #pragma unroll
     for (int u = 0; u < 8; u++) {
-      g += static_cast<int32_t>(v[u] >> 32);
-      h += static_cast<uint32_t>(v[u]);
+      int32_t gv, hv;
+      unpack_pair(v[u], gv, hv);
+      g += gv;
+      h += hv;
     }
   }
   for (; i < m; i += step) {
-    const unsigned long long v = src[static_cast<int64_t>(list[i]) * sink.stride];
-    g += static_cast<int32_t>(v >> 32);
-    h += static_cast<uint32_t>(v);
+    int32_t gv, hv;
+    unpack_pair(src[static_cast<int64_t>(list[i]) * sink.stride], gv, hv);
+    g += gv;
+    h += hv;
   }
   I64Pair* dst = hist.at(node, k, bin0 + bin);
   if (step == 1) {
@@ -634,9 +655,7 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
     for (int u = 0; u < kUnroll; u++) {
       if (valid_c & (1u << u)) {
-        const unsigned long long packed =
-          (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
-          static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+        const unsigned long long packed = pack_pair(q_c[u].x, q_c[u].y);
         T xs[VEC];
         if constexpr (VEC == 1) {
           xs[0] = x_c[u];
@@ -1217,9 +1236,7 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
       for (int u = 0; u < kRows; u++) {
         if (valid_c & (1u << u)) {
-          const unsigned long long packed =
-            (static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].x)) << 32) |
-            static_cast<unsigned long long>(static_cast<uint32_t>(q_c[u].y));
+          const unsigned long long packed = pack_pair(q_c[u].x, q_c[u].y);
           int rel[BV];
           unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
@@ -1268,7 +1285,7 @@ __global__ void __launch_bounds__(kHistThreads)
 template <typename T, int VEC, bool kIdentityRows>
 int launch_search(hipStream_t stream, const HistSetup& hs, const HistArgs<T>& a, const HistBatch& b, unsigned grid)
 {
-  static bool attr_set[kMaxDevices] = {};
+  static std::atomic<bool> attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(histogram_kernel<T, VEC, kIdentityRows>, kLdsBudget, attr_set));
   histogram_kernel<T, VEC, kIdentityRows><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const T*>(b.X), b.qgh);
@@ -1286,7 +1303,7 @@ int launch_search_rows(hipStream_t stream, const HistSetup& hs, const HistArgs<T
 template <typename T, int VEC, typename BinT, bool kRagged>
 int launch_bin_rows(hipStream_t stream, const HistSetup& hs, const BinRowsArgs<T>& a, const HistBatch& b, unsigned grid)
 {
-  static bool attr_set[kMaxDevices] = {};
+  static std::atomic<bool> attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(bin_rows_kernel<T, VEC, BinT, kRagged>, kLdsBudget, attr_set));
   bin_rows_kernel<T, VEC, BinT, kRagged><<<grid, kHistThreads, hs.lds_bytes, stream>>>(
     a, static_cast<const T*>(b.X), b.qgh, static_cast<BinT*>(hs.binned));
@@ -1310,7 +1327,7 @@ template <typename BinT, int BV, bool kEmbed, bool kRoot>
 int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
                      const PartialSink& sink)
 {
-  static bool attr_set[kMaxDevices] = {};
+  static std::atomic<bool> attr_set[kMaxDevices] = {};
   LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
   binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
@@ -1537,9 +1554,10 @@ size_t widest_group(const std::vector<int32_t>& groups, BytesOf bytes_of)
 
 }  // namespace
 
-// The small tables hist_prepare sends to the device (feature groups, record layouts) lie next
-// to each other in the workspace. They are gathered in one pinned block per host thread and
-// sent with one copy: every separate small copy costs about 10 us of the stream's time.
+// The small tables hist_prepare sends to the device (feature groups, record layouts) are carved
+// from one block of the workspace that holds nothing else. They are gathered in one pinned
+// buffer per host thread and sent with one copy: every separate small copy costs about 10 us of
+// the stream's time.
 struct Upload {
   struct Item {
     void* dst;
@@ -1551,50 +1569,47 @@ struct Upload {
   {
     if (bytes > 0) items.push_back({dst, src, bytes});
   }
-  // max_slack: bytes that may lie between two tables (the unused tail of a table's
-  // allocation plus the allocator's padding); anything wider means a foreign buffer
-  int send(hipStream_t stream, size_t max_slack)
+  // [block, block + block_bytes) is the part of the workspace set aside for these tables: the one
+  // copy overwrites all of it (zeros between the tables). Items outside it, or no pinned buffer,
+  // and every table travels by itself.
+  int send(hipStream_t stream, void* block, size_t block_bytes)
   {
     if (items.empty()) return LBT_OK;
-    std::sort(items.begin(), items.end(), [](const Item& a, const Item& b) { return a.dst < b.dst; });
-    char* const lo = static_cast<char*>(items.front().dst);
-    char* const hi = static_cast<char*>(items.back().dst) + items.back().bytes;
-    bool together  = static_cast<size_t>(hi - lo) <= (size_t(1) << 20);
-    for (size_t i = 1; i < items.size() && together; i++) {
-      const char* prev_end = static_cast<const char*>(items[i - 1].dst) + items[i - 1].bytes;
-      const char* next     = static_cast<const char*>(items[i].dst);
-      together = next >= prev_end && static_cast<size_t>(next - prev_end) <= max_slack;
+    char* const lo = static_cast<char*>(block);
+    bool together  = block != nullptr && block_bytes > 0 && block_bytes <= (size_t(1) << 22);
+    for (const Item& it : items) {
+      const char* d = static_cast<const char*>(it.dst);
+      together      = together && d >= lo && d + it.bytes <= lo + block_bytes;
     }
-    static thread_local char* stage          = nullptr;
-    static thread_local size_t stage_bytes   = 0;
-    static thread_local hipEvent_t stage_free = nullptr;
+    ThreadResources& tr = thread_resources();
     if (together) {
-      const size_t total = static_cast<size_t>(hi - lo);
-      if (stage_free == nullptr) {
-        if (hipEventCreateWithFlags(&stage_free, hipEventDisableTiming) != hipSuccess) together = false;
+      if (tr.stage_free == nullptr) {
+        if (hipEventCreateWithFlags(&tr.stage_free, hipEventDisableTiming) != hipSuccess) together = false;
       } else {
-        // the block may still be the source of an earlier call's copy (on another stream)
-        LBT_HIP(hipEventSynchronize(stage_free));
+        // the buffer may still be the source of an earlier call's copy (on another stream)
+        LBT_HIP(hipEventSynchronize(tr.stage_free));
       }
-      if (together && stage_bytes < total) {
-        if (stage != nullptr) LBT_HIP(hipHostFree(stage));
-        stage       = nullptr;
-        stage_bytes = 0;
-        if (hipHostMalloc(reinterpret_cast<void**>(&stage), total + 4096, hipHostMallocDefault) == hipSuccess)
-          stage_bytes = total + 4096;
+      if (together && tr.stage_bytes < block_bytes) {
+        if (tr.stage != nullptr) LBT_HIP(hipHostFree(tr.stage));
+        tr.stage       = nullptr;
+        tr.stage_bytes = 0;
+        if (hipHostMalloc(reinterpret_cast<void**>(&tr.stage), block_bytes + 4096, hipHostMallocDefault) == hipSuccess)
+          tr.stage_bytes = block_bytes + 4096;
         else
           together = false;
       }
       if (together) {
-        std::memset(stage, 0, total);
-        for (const Item& it : items) std::memcpy(stage + (static_cast<char*>(it.dst) - lo), it.src, it.bytes);
-        LBT_HIP(hipMemcpyAsync(lo, stage, total, hipMemcpyHostToDevice, stream));
-        LBT_HIP(hipEventRecord(stage_free, stream));
+        std::memset(tr.stage, 0, block_bytes);
+        for (const Item& it : items) std::memcpy(tr.stage + (static_cast<char*>(it.dst) - lo), it.src, it.bytes);
+        LBT_HIP(hipMemcpyAsync(lo, tr.stage, block_bytes, hipMemcpyHostToDevice, stream));
+        LBT_HIP(hipEventRecord(tr.stage_free, stream));
         items.clear();
         return LBT_OK;
       }
     }
+    // pageable sources that the caller reuses: the copies must have read them before this returns
     for (const Item& it : items) LBT_HIP(hipMemcpyAsync(it.dst, it.src, it.bytes, hipMemcpyHostToDevice, stream));
+    LBT_HIP(hipStreamSynchronize(stream));
     items.clear();
     return LBT_OK;
   }
@@ -1643,8 +1658,8 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
   auto hist_bytes = [&](int f) { return static_cast<size_t>(rp[f + 1] - rp[f]) * 8; };
 
   // search groups: as few as the LDS allows with the smallest table ...
-  // the host arrays below feed asynchronous copies: they persist until the thread's next call,
-  // which starts after this one has synchronised the stream
+  // host copies of the tables; Upload::send has read them when it returns (it copies them into
+  // the thread's pinned buffer, or waits for the copies that read them directly)
   static thread_local std::vector<int32_t> sgroups, groups, stride, tail;
   static thread_local std::vector<int64_t> base;
   static thread_local std::vector<RecInfo> rec;
@@ -1781,8 +1796,7 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     up.add(hs.bin_stride, stride.data(), sizeof(int32_t) * F);
     up.add(hs.bin_tail, tail.data(), sizeof(int32_t) * F);
   }
-  // the tables are allocated one behind the other, each with room for F entries of up to 24 bytes
-  LBT_TRY(up.send(stream, static_cast<size_t>(F) * sizeof(RecInfo) + 512));
+  LBT_TRY(up.send(stream, hs.upload_block, hs.upload_bytes));
   ProfScope ps(LBT_PROF_PROPOSALS, stream);
   if (is_f64)
     build_cells_kernel<double><<<F, 256, 0, stream>>>(static_cast<const double*>(proposals), row_pointers, cells,

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstddef>
 #include <cstdint>
@@ -123,6 +124,25 @@ struct ProfScope {
     if (on) profiler().end(s);
   }
 };
+
+// ---------------------------------------------------------------- host-side state
+//
+// What a host thread keeps between calls, besides its error string: pinned buffers and events
+// that would cost more to create per call than the calls they serve. Created on first use by
+// the thread that calls lbt_build_tree, released by lbt_release_thread_resources() on that
+// thread (or never: a thread that ends without calling it leaves them to the process's end).
+struct ThreadResources {
+  // what the host reads back in the middle of a build (bin counts per feature, the quantiser's
+  // overflow flag): [4 + capacity] ints, two 64-bit statistics first
+  int32_t* mirror        = nullptr;
+  size_t mirror_capacity = 0;
+  hipEvent_t counts_here = nullptr, stats_here = nullptr;
+  // staging buffer of the small tables a build sends to the device, and the event behind its copy
+  char* stage           = nullptr;
+  size_t stage_bytes    = 0;
+  hipEvent_t stage_free = nullptr;
+};
+ThreadResources& thread_resources();
 
 // ---------------------------------------------------------------- device math
 
@@ -251,14 +271,14 @@ __device__ inline bool compute_histogram_bin(int node, const I64Pair* node_sums,
 // (one flag per device ordinal). Setting it twice from two threads is harmless.
 constexpr int kMaxDevices = 64;
 template <typename KernelT>
-int allow_dynamic_lds(KernelT kernel, size_t bytes, bool (&done)[kMaxDevices])
+int allow_dynamic_lds(KernelT kernel, size_t bytes, std::atomic<bool> (&done)[kMaxDevices])
 {
   int device = 0;
   LBT_HIP(hipGetDevice(&device));
-  if (device >= 0 && device < kMaxDevices && done[device]) return LBT_OK;
+  if (device >= 0 && device < kMaxDevices && done[device].load(std::memory_order_acquire)) return LBT_OK;
   LBT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                               static_cast<int>(bytes)));
-  if (device >= 0 && device < kMaxDevices) done[device] = true;
+  if (device >= 0 && device < kMaxDevices) done[device].store(true, std::memory_order_release);
   return LBT_OK;
 }
 
@@ -354,6 +374,10 @@ struct HistSetup {
   // position updates (null: not wanted)
   void* bins_t           = nullptr;
   int64_t bins_t_stride  = 0;      // elements between consecutive features (multiple of 128)
+  // the part of the workspace that holds groups, sgroups, bin_base, bin_stride, bin_tail and rec
+  // (and nothing else): hist_prepare fills it with one copy
+  void* upload_block   = nullptr;
+  size_t upload_bytes  = 0;
   int rpp              = 0;        // rows per workgroup pass, search / binning kernel
   int brpp             = 0;        // rows per workgroup pass, histogram kernel on cached bins
 };

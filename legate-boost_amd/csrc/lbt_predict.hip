@@ -601,14 +601,14 @@ int run_tiled(hipStream_t stream, const T* X, int64_t N, const lbt_packed_ensemb
   const int tile_rows = kTileThreads / lanes;
   ProfScope ps(LBT_PROF_PREDICT, stream, static_cast<double>(N) * (static_cast<double>(F) * sizeof(T) + K * 8.0));
   const unsigned tiles = static_cast<unsigned>((N + tile_rows - 1) / tile_rows);
-  auto launch = [&](auto kernel, bool (&flags)[kMaxDevices]) -> int {
+  auto launch = [&](auto kernel, std::atomic<bool> (&flags)[kMaxDevices]) -> int {
     LBT_TRY(allow_dynamic_lds(kernel, kTileLds, flags));
     kernel<<<tiles, kTileThreads, static_cast<size_t>(ens.lds_bytes), stream>>>(X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes,
                                                       lay.leaves, K, out);
     return LBT_OK;
   };
-  static bool attr[6][kMaxDevices] = {};
-  static bool attr_few[6][kMaxDevices] = {};
+  static std::atomic<bool> attr[6][kMaxDevices] = {};
+  static std::atomic<bool> attr_few[6][kMaxDevices] = {};
   const bool single = K == 1;
   if (ens.few_trees == 1) {
     if (lanes == 4)

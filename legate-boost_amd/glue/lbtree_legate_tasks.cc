@@ -12,6 +12,7 @@
 //   PredictTask::gpu_variant    replaces src/models/tree/predict.cu:26-91
 //   UpdateTreeTask::gpu_variant is new (the reference has a CPU variant only,
 //                               src/models/tree/update_tree.cc:36-133)
+#include <hip/hip_runtime_api.h>
 #include <legate.h>
 
 #include <stdexcept>
@@ -39,15 +40,55 @@ int x_dtype(const legate::PhysicalStore& X)
   throw std::runtime_error("lbtree: X must be float32 or float64");
 }
 
-// Dense, C-ordered instances only (the mapper requests exactly that for these tasks,
-// src/mapper.cc:49-58): the pointer of the first element is then all the library needs.
+// The library reads plain row-major arrays, so the binding checks what the reference checks with
+// EXPECT_DENSE_ROW_MAJOR (src/cpp_utils/cpp_utils.h:139-156) before it hands a pointer over: the
+// instance must be C-ordered over the dimensions that carry data. BUILD_TREE promotes X along
+// dimension 2 and g, h along dimension 1 (legateboost/models/tree.py:117-119); a promoted
+// dimension has stride 0 and is named in `promoted` so that it is left out of the comparison
+// (-1: none). The mapper asks for exactly such instances (src/mapper.cc:49-58); anything else
+// throws, as in the reference, instead of being read with the wrong pitch.
+// Legion's ptr(rect, strides) reports strides in elements.
 template <typename T, int DIM>
-const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
+const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape, int promoted = -1)
 {
   *shape = s.shape<DIM>();
   if (shape->empty()) return nullptr;
   size_t strides[DIM];
   const T* p = s.read_accessor<T, DIM>().ptr(*shape, strides);
+  size_t expected = 1;
+  for (int d = DIM - 1; d >= 0; d--) {
+    if (d == promoted) continue;
+    const size_t extent = static_cast<size_t>(shape->hi[d] - shape->lo[d] + 1);
+    if (extent > 1 && strides[d] != expected)
+      throw std::runtime_error("lbtree: expected a dense row major store (dimension " + std::to_string(d) +
+                               " has stride " + std::to_string(strides[d]) + ", expected " +
+                               std::to_string(expected) + ")");
+    expected *= extent;
+  }
+  return p;
+}
+
+// EXPECT_AXIS_ALIGNED (src/cpp_utils/cpp_utils.h:98-108): two stores cover the same index range
+// along `axis`, so that row i of one is row i of the other.
+template <int DA, int DB>
+void expect_axis_aligned(int axis, const legate::Rect<DA>& a, const legate::Rect<DB>& b)
+{
+  if (a.lo[axis] != b.lo[axis] || a.hi[axis] != b.hi[axis])
+    throw std::runtime_error("lbtree: inconsistent axis alignment (axis " + std::to_string(axis) + ")");
+}
+
+template <typename T, int DIM>
+T* dense_out(legate::PhysicalStore store)
+{
+  auto shape = store.shape<DIM>();
+  size_t strides[DIM];
+  T* p = store.write_accessor<T, DIM>().ptr(shape, strides);
+  size_t expected = 1;
+  for (int d = DIM - 1; d >= 0; d--) {
+    const size_t extent = static_cast<size_t>(shape.hi[d] - shape.lo[d] + 1);
+    if (extent > 1 && strides[d] != expected) throw std::runtime_error("lbtree: expected a dense row major output store");
+    expected *= extent;
+  }
   return p;
 }
 
@@ -58,13 +99,20 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   const auto X_store = context.input(0).data();
   legate::Rect<3> xs, gs, hs;
   const int dtype    = x_dtype(X_store);
-  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
-                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
-  const double* g    = dense_in<double, 3>(context.input(1).data(), &gs);
-  const double* h    = dense_in<double, 3>(context.input(2).data(), &hs);
+  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs, 2))
+                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs, 2));
+  const double* g    = dense_in<double, 3>(context.input(1).data(), &gs, 1);
+  const double* h    = dense_in<double, 3>(context.input(2).data(), &hs, 1);
   const int64_t rows = std::max<int64_t>(xs.hi[0] - xs.lo[0] + 1, 0);
   const int features = static_cast<int>(xs.hi[1] - xs.lo[1] + 1);
   const int outputs  = static_cast<int>(gs.hi[2] - gs.lo[2] + 1);
+  // the checks of build_tree.cu:1282-1289
+  if (gs.lo[2] != 0) throw std::runtime_error("lbtree: outputs should not be split between workers");
+  expect_axis_aligned(0, xs, gs);
+  expect_axis_aligned(0, gs, hs);
+  expect_axis_aligned(1, gs, hs);
+  expect_axis_aligned(2, gs, hs);
+  if (xs.lo[1] != 0) throw std::runtime_error("lbtree: features should not be split between workers");
 
   lbt_build_params p{};
   p.max_depth         = context.scalars().at(0).value<int>();
@@ -84,19 +132,11 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   }
 
   // outputs 0..4: leaf, feature, split, gain, hessian (build_tree.cu:830-842)
-  auto out_ptr = [&](int i, auto tag, auto dim) {
-    using T          = decltype(tag);
-    constexpr int D  = decltype(dim)::value;
-    auto store       = context.output(i).data();
-    auto shape       = store.template shape<D>();
-    size_t strides[D];
-    return store.template write_accessor<T, D>().ptr(shape, strides);
-  };
-  double* leaf     = out_ptr(0, double{}, std::integral_constant<int, 2>{});
-  int32_t* feature = out_ptr(1, int32_t{}, std::integral_constant<int, 1>{});
-  double* split    = out_ptr(2, double{}, std::integral_constant<int, 1>{});
-  double* gain     = out_ptr(3, double{}, std::integral_constant<int, 1>{});
-  double* hessian  = out_ptr(4, double{}, std::integral_constant<int, 2>{});
+  double* leaf     = dense_out<double, 2>(context.output(0).data());
+  int32_t* feature = dense_out<int32_t, 1>(context.output(1).data());
+  double* split    = dense_out<double, 1>(context.output(2).data());
+  double* gain     = dense_out<double, 1>(context.output(3).data());
+  double* hessian  = dense_out<double, 2>(context.output(4).data());
 
   // task-scoped scratch from Legate's pool, as the reference takes its buffers
   // (build_tree.cu:790-794, :880-933, :997); the task already declares allocations
@@ -117,15 +157,19 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   const auto X_store = context.input(0).data();
   legate::Rect<3> xs;
   const int dtype    = x_dtype(X_store);
-  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
-                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
+  // X is promoted along dimension 2, the prediction along dimension 1 (tree.py:256-262)
+  const void* X      = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs, 2))
+                                        : static_cast<const void*>(dense_in<double, 3>(X_store, &xs, 2));
   const int64_t rows = xs.hi[0] - xs.lo[0] + 1;
   if (rows < 1) return;
   auto pred          = context.output(0).data();
   auto pred_shape    = pred.shape<3>();
+  expect_axis_aligned(0, xs, pred_shape);  // predict.cu:56-60
   size_t strides[3];
   double* out       = pred.write_accessor<double, 3>().ptr(pred_shape, strides);
   const int outputs = static_cast<int>(pred_shape.hi[2] - pred_shape.lo[2] + 1);
+  if ((rows > 1 && strides[0] != static_cast<size_t>(outputs)) || (outputs > 1 && strides[2] != 1))
+    throw std::runtime_error("lbtree: expected a dense row major prediction store");
 
   // inputs 1.. are (leaf, feature, split) per tree (legateboost/models/tree.py:264-273)
   std::vector<const double*> leaf, split;
@@ -148,7 +192,13 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   check(lbt_predict(context.get_task_stream(), X, dtype, rows, static_cast<int>(xs.hi[1] - xs.lo[1] + 1),
                     static_cast<int>(leaf.size()), leaf.data(), feature.data(), split.data(), nodes.data(), outputs,
                     out, workspace.ptr(0), ws_bytes));
-  // the buffer is task-scoped: Legate frees it once the work enqueued on the task stream is done
+  // lbt_predict only enqueues; the kernels still read the workspace when this function returns.
+  // Whether Legate keeps a task-scoped buffer alive until the task stream has drained could not
+  // be checked without a Legate build, so the binding waits before it lets go of the buffer, as
+  // the reference's variants do before they return (predict.cu:88, build_tree.cu:1356).
+  if (hipStreamSynchronize(context.get_task_stream()) != hipSuccess)
+    throw std::runtime_error("lbtree: hipStreamSynchronize failed after lbt_predict");
+  workspace.destroy();
 }
 
 /*static*/ void UpdateTreeTask::gpu_variant(legate::TaskContext context)
@@ -157,10 +207,15 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
   legate::Rect<3> xs, gs, hs;
   legate::Rect<1> fs, ss;
   const int dtype        = x_dtype(X_store);
-  const void* X          = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs))
-                                            : static_cast<const void*>(dense_in<double, 3>(X_store, &xs));
-  const double* g        = dense_in<double, 3>(context.input(1).data(), &gs);
-  const double* h        = dense_in<double, 3>(context.input(2).data(), &hs);
+  const void* X          = dtype == LBT_F32 ? static_cast<const void*>(dense_in<float, 3>(X_store, &xs, 2))
+                                            : static_cast<const void*>(dense_in<double, 3>(X_store, &xs, 2));
+  const double* g        = dense_in<double, 3>(context.input(1).data(), &gs, 1);
+  const double* h        = dense_in<double, 3>(context.input(2).data(), &hs, 1);
+  expect_axis_aligned(0, xs, gs);  // update_tree.cc:47-52
+  expect_axis_aligned(0, gs, hs);
+  expect_axis_aligned(1, gs, hs);
+  expect_axis_aligned(2, gs, hs);
+  if (gs.lo[2] != 0) throw std::runtime_error("lbtree: expect all outputs to be present");
   const int32_t* feature = dense_in<int32_t, 1>(context.input(3).data(), &fs);
   const double* split    = dense_in<double, 1>(context.input(4).data(), &ss);
   const int64_t rows     = std::max<int64_t>(xs.hi[0] - xs.lo[0] + 1, 0);
@@ -171,9 +226,8 @@ const T* dense_in(const legate::PhysicalStore& s, legate::Rect<DIM>* shape)
 
   auto leaf_store = context.output(0).data();
   auto hess_store = context.output(1).data();
-  size_t strides[2];
-  double* leaf    = leaf_store.write_accessor<double, 2>().ptr(leaf_store.shape<2>(), strides);
-  double* hessian = hess_store.write_accessor<double, 2>().ptr(hess_store.shape<2>(), strides);
+  double* leaf    = dense_out<double, 2>(leaf_store);
+  double* hessian = dense_out<double, 2>(hess_store);
 
   const size_t ws_bytes = lbt_update_tree_workspace_bytes(rows, outputs, nodes);
   auto workspace        = legate::create_buffer<int8_t>(ws_bytes, legate::Memory::GPU_FB_MEM, 256);

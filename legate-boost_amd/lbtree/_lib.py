@@ -97,6 +97,8 @@ def _load():
     lib = C.CDLL(SO_PATH)
     lib.lbt_last_error.restype = C.c_char_p
     lib.lbt_version.restype = C.c_int
+    lib.lbt_release_thread_resources.restype = C.c_int
+    lib.lbt_release_thread_resources.argtypes = []
     lib.lbt_build_tree_workspace_bytes.restype = C.c_size_t
     lib.lbt_build_tree_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32,
                                                    C.c_int64]
@@ -154,7 +156,7 @@ def _load():
 lib = _load()
 
 EXPORTS = [
-    "lbt_last_error", "lbt_version", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_build_tree_async", "lbt_predict",
+    "lbt_last_error", "lbt_version", "lbt_release_thread_resources", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_build_tree_async", "lbt_predict",
     "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_select_split_samples_workspace_bytes", "lbt_select_split_samples",

@@ -488,6 +488,7 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
       memcpy(taps->positions_per_level + (size_t)depth * N * 2, pos, sizeof(int32_t) * 2 * (size_t)N);
     int64_t lvl_inst = 0, lvl_built_inst = 0;
     int32_t lvl_built_nodes = 0;
+    int last_built_node     = -1;
 
     /* PrepareBatches, build_tree.cu:1207-1258 */
     const int64_t nodes_in_level = (int64_t)1 << depth;
@@ -537,6 +538,11 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
         if (!compute_histogram_bin(node, node_sums, K, hist_contains_node(&hs, parent_of(node))))
           continue;
         lvl_built_inst++;
+        /* the order is sorted by node: a node that is built and holds rows is counted at its first row */
+        if (node != last_built_node) {
+          lvl_built_nodes++;
+          last_built_node = node;
+        }
         for (int f = 0; f < F; f++) {
           int b = bins[(int64_t)row * F + f];
           for (int k = 0; k < K; k++) {
@@ -551,7 +557,6 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
       for (int node = batch_begin; node < batch_end; node++) {
         int par = parent_of(node);
         int built = compute_histogram_bin(node, node_sums, K, hist_contains_node(&hs, par));
-        if (built && node_sums[((int64_t)node * K + 0) * 2 + 1] > 0) lvl_built_nodes++;
         for (int k = 0; k < K; k++) {
           if (node_sums[((int64_t)node * K + k) * 2 + 1] <= 0) continue;
           if (!built) continue;

@@ -115,7 +115,7 @@ typedef struct {
   int32_t hist_node_begin; /* out */
   int32_t hist_node_end;   /* out */
   /* per depth: instances in all batches, instances whose node was built,
-   * number of nodes built (for byte accounting). [max_depth] each. */
+   * number of built nodes that hold at least one row (for byte accounting). [max_depth] each. */
   int64_t* level_instances;
   int64_t* level_built_instances;
   int32_t* level_built_nodes;

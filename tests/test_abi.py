@@ -24,7 +24,8 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(_lib.lib, n), n
     assert sorted(_lib.EXPORTS) == names
-    assert _lib.lib.lbt_version() >= 1
+    assert _lib.lib.lbt_version() >= 2
+    assert _lib.lib.lbt_release_thread_resources() == 0  # nothing held yet: nothing to do, no GPU call
 
 
 def test_workspace_query():

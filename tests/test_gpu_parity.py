@@ -60,6 +60,58 @@ def test_depth_zero_and_regularisation_variants():
         gu.assert_tree_parity(gr, cr)
 
 
+@pytest.mark.parametrize("n,f,k,depth,s", [(30000, 20, 1, 6, 256), (20000, 70, 2, 5, 64), (9000, 6, 3, 4, 300)])
+def test_negative_hessians_bit_exact(n, f, k, depth, s):
+    """A custom objective may hand over negative hessians; the reference rounds and sums them as
+    int64 like any other value (build_tree.cu:112-129). Embedded and gathered gradient pairs,
+    one- and two-byte bins."""
+    import gpu_util as gu
+
+    X, g, h = _problem(n + k, n, f, k)
+    rs = np.random.RandomState(n)
+    h = np.where(rs.rand(n, k) < 0.15, -h, h)
+    h[:5] = -3.0
+    gr, cr = gu.both(X, g, h, levels=True, max_depth=depth, split_samples=s, seed=99)
+    gu.assert_tree_parity(gr, cr, levels=True)
+    assert (cr.quantised[:, :, 1] < 0).any() and (cr.feature != -1).sum() > 5
+    # all hessians negative: the root's sum is not positive, nothing splits (build_tree.cu:712)
+    gr, cr = gu.both(X, g, -np.abs(h), max_depth=3, split_samples=s, seed=5)
+    gu.assert_tree_parity(gr, cr)
+    assert (cr.feature == -1).all()
+
+
+@pytest.mark.parametrize("wait", [True, False])
+def test_error_raised_inside_a_build_reaches_the_caller(wait):
+    """One entry holds the whole absolute gradient sum and the stochastic rounding takes it up to
+    2^31 (seed, row and value chosen for that: the oracle confirms the value), which the packed
+    32-bit pairs cannot hold. The library notices after the first level is queued: the call must
+    return the status, the synchronising form with the stream drained, and later calls work."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import _lib, ops
+
+    n, seed, row = 4096, 308, 1068
+    g = np.zeros((n, 1))
+    g[row, 0] = 4.236547993389047
+    h = np.zeros((n, 1))
+    h[0, 0] = 1.0
+    q = orc.quantise_all(g, h, seed, orc.scales(orc.abs_sums(g, h)))
+    assert q[row, 0, 0] == 2 ** 31
+    X, _, _ = _problem(3, n, 7, 1)
+    with pytest.raises(_lib.LbtError, match="2\\^31"):
+        ops.build_tree(X, g, h, max_depth=4, split_samples=32, seed=seed, wait=wait)
+    if wait:
+        assert torch.cuda.current_stream().query()  # nothing of the failed call is still queued
+    torch.cuda.synchronize()
+    # the same thread and workspace serve the next call, also after the thread's pinned buffers
+    # and events have been released
+    X2, g2, h2 = _problem(4, n, 7, 1)
+    for _ in range(2):
+        gr, cr = gu.both(X2, g2, h2, max_depth=4, split_samples=32, seed=seed)
+        gu.assert_tree_parity(gr, cr)
+        assert _lib.lib.lbt_release_thread_resources() == 0
+
+
 def test_feature_set():
     import gpu_util as gu
 
