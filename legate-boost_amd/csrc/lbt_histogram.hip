@@ -395,6 +395,47 @@ __device__ inline void merge_sub_histogram(unsigned long long* s_hist, int nb, I
   }
 }
 
+// The striped layout of the packed sub-histogram: word bin * W + p holds bin `bin` of the group's
+// feature p, W a power of two (at least 16) that is not smaller than the group. The LDS serves a
+// wave-level 64-bit atomic quarter wave by quarter wave, and the 16 lanes of a quarter conflict
+// when two of them fall on the same pair of banks, i.e. when their word indices agree modulo 16.
+// Here the index modulo 16 is the feature modulo 16, whatever the bin is, and a lane that holds
+// 16 bins of a row takes them in an order of its own, byte (step + lane) mod 16 at every step:
+// the 16 lanes of a quarter wave then always work on 16 different features modulo 16 and never
+// conflict (7 cycles per wave-level atomic where data-dependent banks cost 10 to 11 and, with
+// the same-address collisions of the 16 rows of a wave, 15 to 16 in the kernel).
+struct Stripes {
+  int log_w;  // log2 W; negative: the layout is [feature][bin], one run of bins per feature
+  int bins;   // bins of the widest feature (rows of the striped array)
+  __host__ __device__ int words() const { return bins << log_w; }
+};
+
+// Merge of a striped sub-histogram into the int64 histogram of a node; s_off[p] is the place of
+// feature p's first bin in the group's run of bins.
+// sole_owner: no other workgroup adds to these bins and nothing has been added to them yet (the
+// histogram starts from zero and the parked parts of a node are added after the launch): the
+// sums are stored as they are, which neither waits for a load nor occupies the L2's atomic units.
+__device__ inline void merge_striped(unsigned long long* s_hist, const Stripes& st, const int* s_off, I64Pair* dst,
+                                     bool sole_owner)
+{
+  const int words = st.words();
+  for (int i = threadIdx.x; i < words; i += kHistThreads) {
+    const unsigned long long v = s_hist[i];
+    if (v != 0) {
+      int32_t gv, hv;
+      unpack_pair(v, gv, hv);
+      I64Pair* d = dst + s_off[i & ((1 << st.log_w) - 1)] + (i >> st.log_w);
+      if (sole_owner) {
+        *d = I64Pair{gv, hv};
+      } else {
+        if (gv != 0) atomic_add_i64(&d->grad, static_cast<int64_t>(gv));
+        if (hv != 0) atomic_add_i64(&d->hess, static_cast<int64_t>(hv));
+      }
+      s_hist[i] = 0;
+    }
+  }
+}
+
 // Where the workgroups of a launch park their sub-histograms for reduce_partials_kernel.
 struct PartialSink {
   unsigned long long* partials;
@@ -411,19 +452,22 @@ struct PartialSink {
 // clears them; a pass after the launch adds up the slots of every (node, group, output) with
 // plain loads. Without a free slot the atomics do it. All threads of the workgroup call this.
 __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst, const PartialSink& sink,
-                                          int tag, int* s_slot, bool sole_owner)
+                                          int tag, int* s_slot, bool sole_owner, const Stripes& st, const int* s_off)
 {
+  if (sole_owner && st.log_w >= 0) {
+    merge_striped(s_hist, st, s_off, dst, true);
+    return;
+  }
   if (sole_owner) {
-    // every row of the node went through this workgroup: nobody else adds to these bins
+    // every row of the node went through this workgroup: nobody else adds to these bins, and
+    // nothing has been added to them yet (the histogram starts from zero, parked parts of the
+    // node are added after the launch), so the sums are stored as they are
     for (int i = threadIdx.x; i < nb; i += kHistThreads) {
       const unsigned long long v = s_hist[i];
       if (v != 0) {
         int32_t gv, hv;
         unpack_pair(v, gv, hv);
-        I64Pair p = dst[i];
-        p.grad += gv;
-        p.hess += hv;
-        dst[i]    = p;
+        dst[i]    = I64Pair{gv, hv};
         s_hist[i] = 0;
       }
     }
@@ -447,11 +491,15 @@ __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I6
     slot = *s_slot;
   }
   if (slot < sink.slots) {
+    // the words as they lie in the LDS (striped: all of the array)
+    const int words         = st.log_w >= 0 ? st.words() : nb;
     unsigned long long* out = sink.partials + static_cast<int64_t>(slot) * sink.stride;
-    for (int i = threadIdx.x; i < nb; i += kHistThreads) {
+    for (int i = threadIdx.x; i < words; i += kHistThreads) {
       out[i]    = s_hist[i];
       s_hist[i] = 0;
     }
+  } else if (st.log_w >= 0) {
+    merge_striped(s_hist, st, s_off, dst, false);
   } else {
     merge_sub_histogram(s_hist, nb, dst);
   }
@@ -464,7 +512,7 @@ __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I6
 // the levels near the root) adds them with atomics. Integer sums: any order gives the same.
 __global__ void __launch_bounds__(kHistThreads)
   reduce_partials_kernel(PartialSink sink, int K, int n_groups, const int32_t* __restrict__ groups,
-                         const int32_t* __restrict__ row_pointers, HistView hist, int first_node)
+                         const int32_t* __restrict__ row_pointers, HistView hist, int first_node, Stripes st)
 {
   const int tag = blockIdx.y;
   const int m   = min(sink.list_count[tag], kPartialListCap);
@@ -473,10 +521,20 @@ __global__ void __launch_bounds__(kHistThreads)
   const int node  = first_node + tag / n_gk;
   const int gk    = tag - tag / n_gk * n_gk;
   const int group = gk / K, k = gk - gk / K * K;
-  const int bin0  = row_pointers[groups[group]];
+  int bin0        = row_pointers[groups[group]];
   const int nb    = row_pointers[groups[group + 1]] - bin0;
+  // `bin` is the word of the parked image; out_bin its place in the group's run of bins
   const int bin   = blockIdx.x * kHistThreads + threadIdx.x;
-  if (bin >= nb) return;
+  int out_bin     = bin;
+  if (st.log_w >= 0) {
+    if (bin >= st.words()) return;
+    const int f = groups[group] + (bin & ((1 << st.log_w) - 1));
+    const int b = bin >> st.log_w;
+    if (f >= groups[group + 1] || b >= row_pointers[f + 1] - row_pointers[f]) return;
+    out_bin = row_pointers[f] - bin0 + b;
+  } else if (bin >= nb) {
+    return;
+  }
   const int32_t* __restrict__ list = sink.lists + static_cast<int64_t>(tag) * kPartialListCap;
   const unsigned long long* src    = sink.partials + bin;
   const int step                   = gridDim.z;
@@ -501,7 +559,7 @@ __global__ void __launch_bounds__(kHistThreads)
     g += gv;
     h += hv;
   }
-  I64Pair* dst = hist.at(node, k, bin0 + bin);
+  I64Pair* dst = hist.at(node, k, bin0 + out_bin);
   if (step == 1) {
     dst->grad += g;
     dst->hess += h;
@@ -1020,7 +1078,19 @@ struct BinnedArgs {
   const int32_t* row_pointers;
   const int32_t* groups;
   HistView hist;
+  Stripes stripes;  // layout of the LDS sub-histogram
 };
+
+// The 16 bytes of `w` rotated down by t bytes: byte v of the result is byte (v + t) mod 16 of w.
+__device__ __forceinline__ uint4 rotate_bytes(const uint4& w, int t)
+{
+  const bool r1 = (t & 4) != 0, r2 = (t & 8) != 0;
+  const uint32_t x1 = r1 ? w.y : w.x, y1 = r1 ? w.z : w.y, z1 = r1 ? w.w : w.z, w1 = r1 ? w.x : w.w;
+  const uint32_t x2 = r2 ? z1 : x1, y2 = r2 ? w1 : y1, z2 = r2 ? x1 : z1, w2 = r2 ? y1 : w1;
+  const uint32_t b = static_cast<uint32_t>(t) & 3u;
+  return make_uint4(__builtin_amdgcn_alignbyte(y2, x2, b), __builtin_amdgcn_alignbyte(z2, y2, b),
+                    __builtin_amdgcn_alignbyte(w2, z2, b), __builtin_amdgcn_alignbyte(x2, w2, b));
+}
 
 // 4 x 4 byte transpose: input word r is row r and its byte b is feature b; output word b holds
 // feature b of rows 0..3.
@@ -1042,13 +1112,19 @@ __device__ __forceinline__ void turn_bytes(uint32_t w0, uint32_t w1, uint32_t w2
 // takes four consecutive rows per tile and, besides accumulating, stores their bins feature by
 // feature into bins_t ([feature][row]), which the position updates read: the feature-major copy
 // costs no second pass over the cache.
-template <typename BinT, int BV, bool kEmbed, bool kRoot>
+// kStriped (one-byte bins): the LDS sub-histogram is striped (see Stripes) and every lane takes the
+// 16 bins of a row in its own rotated order.
+constexpr int kStripeMaxW = 256;  // widest group the striped layout serves, in features
+
+template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped>
 __global__ void __launch_bounds__(kHistThreads)
   binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
                           const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride,
                           int32_t* pair_sync, PartialSink sink)
 {
+  static_assert(!kStriped || BV == 16, "the striped layout is built for lanes that hold 16 one-byte bins");
   __shared__ int s_slot;
+  __shared__ int s_off[kStriped ? kStripeMaxW : 1];  // striped: first bin of every feature in the group's run of bins
   using Word = typename BinVec<BinT, BV>::type;
   constexpr int kRows = kRoot ? 4 : (BV == 16 ? kBinnedUnroll / 2 : kBinnedUnroll);  // rows per lane and tile
   extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
@@ -1064,9 +1140,16 @@ __global__ void __launch_bounds__(kHistThreads)
   const int bin0 = a.row_pointers[f0];
   const int nb   = a.row_pointers[f1] - bin0;
   unsigned long long* s_hist = reinterpret_cast<unsigned long long*>(smem_raw);
-  // behind the group's bins every lane owns a spare slot that takes the adds of its features
-  // past the group end (never read; private, so these adds do not collide)
-  for (int i = threadIdx.x; i < nb + kHistThreads; i += kHistThreads) s_hist[i] = 0;
+  const Stripes st           = a.stripes;
+  if constexpr (kStriped) {
+    for (int i = threadIdx.x; i < st.words(); i += kHistThreads) s_hist[i] = 0;
+    for (int i = threadIdx.x; i < (1 << st.log_w); i += kHistThreads)
+      s_off[i] = i < gs ? a.row_pointers[f0 + i] - bin0 : 0;
+  } else {
+    // behind the group's bins every lane owns a spare slot that takes the adds of its features
+    // past the group end (never read; private, so these adds do not collide)
+    for (int i = threadIdx.x; i < nb + kHistThreads; i += kHistThreads) s_hist[i] = 0;
+  }
 
   const RecInfo ri        = a.rec[group];
   const int lanes_per_row = (gs + BV - 1) / BV;
@@ -1079,10 +1162,24 @@ __global__ void __launch_bounds__(kHistThreads)
   const int64_t stride              = ri.stride;
   // the gradient pair may share the last 16 bytes a lane loads as bins: that lane blanks them
   const bool strip = kEmbed && BV == 16 && ri.q_off >= my_off && ri.q_off < my_off + static_cast<int>(sizeof(Word));
+  const int nv = min(BV, max(0, gs - fl));  // features this lane really has
+  // packed layout: first word of every feature of the lane. Striped: the lane's step v works on its
+  // byte (v + rot) mod 16; c_base[v] is the byte offset of that feature's column in the LDS array
+  // and bit v of `has` says whether the lane has that feature.
+  const int rot = threadIdx.x & 15;
+  unsigned has  = 0;
   int c_base[BV];
 #pragma unroll
-  for (int v = 0; v < BV; v++) c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
-  const int nv = min(BV, max(0, gs - fl));  // features this lane really has
+  for (int v = 0; v < BV; v++) {
+    if constexpr (kStriped) {
+      const int o = (v + rot) & 15;
+      c_base[v]   = (fl + o) * 8;
+      has |= o < nv ? (1u << v) : 0u;
+    } else {
+      c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
+    }
+  }
+  const int stripe_shift = st.log_w + 3;  // a bin's row of the striped array, in bytes
   const unsigned long long max_abs = qstats[0];
   const int n_tiles = meta->n_tiles;
   const int t_begin = static_cast<int>(static_cast<int64_t>(n_tiles) * chunk / w.n_chunks);
@@ -1177,7 +1274,7 @@ __global__ void __launch_bounds__(kHistThreads)
         if (cur_node >= 0)
           park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink,
                              (cur_node - w.level_first - w.j0) * w.n_gk + gk, &s_slot,
-                             owners && tc.node != cur_node && node_rows == node_total);
+                             owners && tc.node != cur_node && node_rows == node_total, st, s_off);
         __syncthreads();
         if (tc.node != cur_node) {
           node_rows  = 0;
@@ -1232,6 +1329,11 @@ __global__ void __launch_bounds__(kHistThreads)
         }
       }
     }
+    if constexpr (kStriped) {
+      // from here on a lane's bins stand in its own order (the feature-major copy above took them as loaded)
+#pragma unroll
+      for (int u = 0; u < kRows; u++) b_c[u] = rotate_bytes(b_c[u], rot);
+    }
     if (!direct) {
 #pragma unroll
       for (int u = 0; u < kRows; u++) {
@@ -1242,8 +1344,14 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
           // a lane whose 16 bins reach past the group end leaves those out: an atomic costs by
           // the lanes that take part in it
-          for (int v = 0; v < BV; v++)
-            if (v < nv) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
+          for (int v = 0; v < BV; v++) {
+            if constexpr (kStriped) {
+              if (has & (1u << v))
+                atomicAdd(reinterpret_cast<unsigned long long*>(smem_raw + ((rel[v] << stripe_shift) + c_base[v])), packed);
+            } else {
+              if (v < nv) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
+            }
+          }
         }
       }
     } else {
@@ -1255,8 +1363,16 @@ __global__ void __launch_bounds__(kHistThreads)
           unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
           for (int v = 0; v < BV; v++) {
-            if (fl + v < gs) {
-              const int bin = c_base[v] + rel[v];
+            bool mine;
+            int bin;
+            if constexpr (kStriped) {
+              mine = (has & (1u << v)) != 0;
+              bin  = mine ? s_off[c_base[v] >> 3] + rel[v] : 0;
+            } else {
+              mine = fl + v < gs;
+              bin  = c_base[v] + rel[v];
+            }
+            if (mine) {
               atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
               atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
             }
@@ -1279,7 +1395,7 @@ __global__ void __launch_bounds__(kHistThreads)
   __syncthreads();
   if (cur_node >= 0)
     park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink, (cur_node - w.level_first - w.j0) * w.n_gk + gk,
-                       &s_slot, owners && node_rows == node_total);
+                       &s_slot, owners && node_rows == node_total, st, s_off);
 }
 
 template <typename T, int VEC, bool kIdentityRows>
@@ -1323,13 +1439,15 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
   return launch_bin_rows<T, VEC, uint16_t, false>(stream, hs, a, b, grid);
 }
 
-template <typename BinT, int BV, bool kEmbed, bool kRoot>
+template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped>
 int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
                      const PartialSink& sink)
 {
   static std::atomic<bool> attr_set[kMaxDevices] = {};
-  LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot>, kLdsBudget, attr_set));
-  binned_histogram_kernel<BinT, BV, kEmbed, kRoot><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
+  // the striped kernel keeps a table of feature offsets in static LDS and never asks for more than this
+  LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped>,
+                            kStriped ? kLdsBudget - 8 * 1024 : kLdsBudget, attr_set));
+  binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
     // meeting points only between workgroups that run at the same time: one that waits for a
@@ -1341,8 +1459,14 @@ template <typename BinT, int BV, bool kEmbed>
 int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
                   bool root, const PartialSink& sink)
 {
-  if (root) return launch_binned_as<BinT, BV, kEmbed, true>(stream, hs, a, b, grid, sink);
-  return launch_binned_as<BinT, BV, kEmbed, false>(stream, hs, a, b, grid, sink);
+  if constexpr (BV == 16) {
+    if (a.stripes.log_w >= 0) {
+      if (root) return launch_binned_as<BinT, BV, kEmbed, true, true>(stream, hs, a, b, grid, sink);
+      return launch_binned_as<BinT, BV, kEmbed, false, true>(stream, hs, a, b, grid, sink);
+    }
+  }
+  if (root) return launch_binned_as<BinT, BV, kEmbed, true, false>(stream, hs, a, b, grid, sink);
+  return launch_binned_as<BinT, BV, kEmbed, false, false>(stream, hs, a, b, grid, sink);
 }
 
 // As many resident workgroups as the LDS allows per CU; row-tile ranges come in multiples
@@ -1442,6 +1566,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     a.row_pointers = b.row_pointers;
     a.groups       = hs.groups;
     a.hist         = b.hist;
+    a.stripes      = Stripes{hs.stripe_log, hs.stripe_bins};
     PartialSink sink{hs.partials, hs.partial_lists, hs.partial_list_count, hs.partial_count, 0, hs.partial_stride};
     if (hs.partials != nullptr && static_cast<int64_t>(w.n_nodes) * w.n_gk <= kPartialMaxLists)
       sink.slots = hs.partial_slots;
@@ -1466,7 +1591,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
       const int split      = std::max(1, std::min(16, 256 / (lists * bin_chunks)));
       dim3 rgrid(static_cast<unsigned>(bin_chunks), static_cast<unsigned>(lists), static_cast<unsigned>(split));
       reduce_partials_kernel<<<rgrid, kHistThreads, 0, stream>>>(sink, a.K, w.n_gk / a.K, a.groups, a.row_pointers, a.hist,
-                                                                 w.level_first + w.j0);
+                                                                 w.level_first + w.j0, a.stripes);
     }
     return LBT_OK;
   }
@@ -1751,6 +1876,23 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
     hs.n_groups   = static_cast<int>(groups.size()) - 1;
     hs.blds_bytes = (blds + 8 * kHistThreads + 15) & ~size_t(15);
     hs.partial_stride = static_cast<int>(blds / 8);  // bins of the widest group
+    // The striped layout (one-byte bins) takes max bins x W words, W the power of two that holds the
+    // widest group: used whenever that fits the LDS with the groups the packed layout would have.
+    hs.stripe_log  = -1;
+    hs.stripe_bins = 0;
+    if (hs.bin_bytes == 1) {
+      int widest = 1;
+      for (int g = 0; g < hs.n_groups; g++) widest = std::max(widest, groups[g + 1] - groups[g]);
+      int log_w = 4;
+      while ((1 << log_w) < widest) log_w++;
+      const size_t need = static_cast<size_t>(max_feature_bins) * 8 << log_w;
+      if ((1 << log_w) <= kStripeMaxW && need <= kLdsBudget - 8 * 1024) {
+        hs.stripe_log     = log_w;
+        hs.stripe_bins    = max_feature_bins;
+        hs.blds_bytes     = (need + 15) & ~size_t(15);
+        hs.partial_stride = static_cast<int>(need / 8);
+      }
+    }
     if (hs.partial_stride > kPartialStrideMax) hs.partials = nullptr;
     hs.brpp       = rows_per_pass(groups, hs.bvec);
     up.add(hs.groups, groups.data(), sizeof(int32_t) * groups.size());

@@ -365,6 +365,8 @@ struct HistSetup {
   int bvec             = 1;        // cached bins a lane of the histogram kernel loads at once
   bool embed           = false;    // records carry the row's (grad, hess)
   size_t blds_bytes    = 0;        // LDS of the histogram kernel (packed sub-histogram only)
+  int stripe_log       = -1;       // log2 of the striped layout's row width in features; negative: [feature][bin]
+  int stripe_bins      = 0;        // bins of the widest feature (rows of the striped array)
   RecInfo* rec         = nullptr;  // [n_groups]
   int64_t max_rec_stride = 0;      // widest record, bytes
   int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
