@@ -184,6 +184,25 @@ int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64
                            int64_t row_offset, int32_t seed, int32_t* quantised, int64_t* root_sums, double* scales,
                            void* workspace, size_t workspace_bytes);
 
+/*
+ * lbt_quantise_gradients for callers that cannot allocate device memory or bring a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference. Same arguments and same results, bit for bit, as
+ * lbt_quantise_gradients, without the workspace: the partial sums and counters of the pass live
+ * in a device array inside the library (about 260 KB on every GPU the library runs on, held
+ * until the process ends). The call allocates nothing and frees nothing; its first call on a
+ * device looks up the array's address on that device (hipGetSymbolAddress), later calls reuse it.
+ *   n_rows * n_outputs  at most LBT_QUANTISE_STATIC_MAX_ENTRIES; more is rejected with
+ *                       LBT_ERR_INVALID and a message that names the limit
+ * All calls on one GPU share that GPU's array: two calls that overlap on one GPU (different
+ * streams, or different host threads) race; calls on one stream are ordered. Nothing is
+ * carried over from one call to the next.
+ */
+#define LBT_QUANTISE_STATIC_MAX_ENTRIES (1LL << 26)
+int lbt_quantise_gradients_static(void* stream, const double* g, const double* h, int64_t n_rows,
+                                  int32_t n_outputs, int64_t row_offset, int32_t seed, int32_t* quantised,
+                                  int64_t* root_sums, double* scales);
+
 /* Device scratch for lbt_predict: room for the ensemble packed into one node array and one
  * leaf array (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
 size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype);

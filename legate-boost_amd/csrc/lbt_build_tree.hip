@@ -1876,6 +1876,77 @@ int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64
                             reinterpret_cast<int2*>(quantised), reinterpret_cast<lbt::I64Pair*>(root_sums));
 }
 
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// The quantiser for callers that cannot allocate: its scratch (the partial sums of the two
+// absolute sums and the two statistics words) lives in a device array of this library instead
+// of a caller's workspace. Every GPU the library is loaded on holds its own copy of the array
+// until the process ends. `static_scratch` is only the host-side handle of it: what kernels and
+// copies are given is the address that hipGetSymbolAddress returns for the current device.
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int64_t kStaticMaxEntries = LBT_QUANTISE_STATIC_MAX_ENTRIES;  // n_rows * n_outputs
+// two levels of partial sums (one double per 4096 entries, twice) for g and h, 256-byte pitch, and qstats
+constexpr size_t kStaticScratchBytes =
+  2 * (((static_cast<size_t>(kStaticMaxEntries) / 4096 * sizeof(double)) + 255) / 256 * 256) + 2 * 256 + 256 + 256;
+static __device__ __align__(256) unsigned char static_scratch[kStaticScratchBytes];
+
+std::atomic<void*> static_scratch_ptr[lbt::kMaxDevices] = {};
+
+// The array's address on the current device, resolved once per device.
+int static_scratch_address(void** out)
+{
+  int device = 0;
+  LBT_HIP(hipGetDevice(&device));
+  LBT_REQUIRE(device >= 0 && device < lbt::kMaxDevices, "device ordinal %d is not supported", device);
+  void* p = static_scratch_ptr[device].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    LBT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch)));
+    LBT_REQUIRE(p != nullptr, "the address of the static scratch array is null");
+    static_scratch_ptr[device].store(p, std::memory_order_release);  // two threads resolve the same address
+  }
+  *out = p;
+  return LBT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int lbt_quantise_gradients_static(void* stream, const double* g, const double* h, int64_t n_rows, int32_t n_outputs,
+                                  int64_t row_offset, int32_t seed, int32_t* quantised, int64_t* root_sums,
+                                  double* scales)
+{
+  LBT_REQUIRE(n_rows >= 1 && n_rows < 2147483647LL && n_outputs >= 1 && n_outputs <= 65535, "bad shape");
+  LBT_REQUIRE(n_rows * static_cast<int64_t>(n_outputs) <= kStaticMaxEntries,
+              "lbt_quantise_gradients_static takes at most %lld entries (n_rows * n_outputs), got %lld: use "
+              "lbt_quantise_gradients with a workspace",
+              static_cast<long long>(kStaticMaxEntries), static_cast<long long>(n_rows * static_cast<int64_t>(n_outputs)));
+  LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
+  LBT_REQUIRE(g && h && quantised && root_sums && scales, "null input or output pointer");
+  void* scratch = nullptr;
+  LBT_TRY(static_scratch_address(&scratch));
+  lbt::Arena ar;
+  ar.base = static_cast<char*>(scratch);
+  ar.cap  = kStaticScratchBytes;
+  QuantiserScratch w;
+  make_quantiser_scratch(ar, w, n_rows, n_outputs);
+  if (ar.failed) {
+    lbt::set_error("static scratch too small: %zu bytes, %zu needed", kStaticScratchBytes, ar.used);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  lbt::ProfScope ps(LBT_PROF_QUANTISE, s, static_cast<double>(n_rows) * n_outputs * (16 + 16 + 8));
+  // Nothing of an earlier call's contents is read: every partial sum that is read was written
+  // by this call, and scales_kernel resets the statistics words. The root sums are cleared by a
+  // kernel (a memset node would not replay in a captured graph).
+  lbt::zero_kernel<<<1, lbt::kThreads, 0, s>>>(reinterpret_cast<uint4*>(root_sums), n_outputs);
+  return lbt::run_quantiser(s, g, h, n_rows, n_outputs, row_offset, seed, w.part_a, w.part_b, scales, w.qstats,
+                            reinterpret_cast<int2*>(quantised), reinterpret_cast<lbt::I64Pair*>(root_sums));
+}
+
 int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,
                    int64_t n_rows, int32_t n_features, const double* g, const double* h,
                    int32_t n_outputs, const uint8_t* feature_set, const lbt_build_params* params,

@@ -16,6 +16,7 @@ LBT_F64 = 1
 LBT_MAX_SPLIT_SAMPLES = 2048
 LBT_OBJ_SQUARED_ERROR = 0
 LBT_OBJ_LOG_LOSS = 1
+LBT_QUANTISE_STATIC_MAX_ENTRIES = 1 << 26
 PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "positions", "other", "predict", "binning"]
 
 
@@ -145,6 +146,9 @@ def _load():
     lib.lbt_quantise_gradients.restype = C.c_int
     lib.lbt_quantise_gradients.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64,
                                            C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_quantise_gradients_static.restype = C.c_int
+    lib.lbt_quantise_gradients_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64,
+                                                  C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.lbt_profile_enable.restype = None
     lib.lbt_profile_enable.argtypes = [C.c_int]
     lib.lbt_profile_reset.restype = None
@@ -160,7 +164,7 @@ EXPORTS = [
     "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_select_split_samples_workspace_bytes", "lbt_select_split_samples",
-    "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_profile_enable", "lbt_profile_reset",
+    "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_quantise_gradients_static", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",
 ]
 
