@@ -42,65 +42,84 @@ def parse():
 
 
 def cpu_baseline_build(X_sample, y_sample, max_depth, split_samples, lr, full_rows, seconds, n_outputs_classes=0):
-    """Rounds/s of the restated CPU variant on a row sample, scaled to the full row count."""
+    """Rounds/s of the restated CPU variant of the reference on a row sample, at P = the host threads of this
+    GPU's share of the machine and at P = 1, each scaled to the full row count (the work of a round is linear
+    in the rows: binning, histograms and the position update all walk them once per level)."""
     import numpy as np
 
     import cpu_variant_lib as cv
 
+    # a one-GPU box gives its job 16 host threads whatever os.cpu_count() reports
     cores = max(1, min(16, os.cpu_count() or 1))
     n = X_sample.shape[0]
-    if n_outputs_classes:
-        k = n_outputs_classes
-        pred = np.zeros((n, k))
-    else:
-        k = 1
-        pred = np.full((n, 1), y_sample.mean())
-    rounds = 0
-    t0 = time.perf_counter()
-    while True:
-        if n_outputs_classes:
-            e = np.exp(pred - pred.max(axis=1, keepdims=True))
-            p = e / e.sum(axis=1, keepdims=True)
-            g = p.copy()
-            g[np.arange(n), y_sample.astype(np.int64)] -= 1.0
-            g *= lr
-            h = np.maximum(p * (1 - p), 1e-8)
-        else:
-            g = (pred - y_sample.reshape(-1, 1)) * lr
-            h = np.ones((n, 1))
-        leaf, feat, split, gain, hess = cv.build_tree(X_sample, g, h, max_depth=max_depth,
-                                                      split_samples=split_samples, seed=rounds, n_threads=cores)
-        pred += cv.predict(X_sample, [(leaf, feat, split)], k, n_threads=cores)
-        rounds += 1
-        dt = time.perf_counter() - t0
-        if dt >= seconds and rounds >= 2:
-            break
-    rate_sample = rounds / dt
+    k = n_outputs_classes or 1
+
+    def run(n_threads, budget, min_rounds):
+        pred = np.zeros((n, k)) if n_outputs_classes else np.full((n, 1), y_sample.mean())
+        rounds = 0
+        t0 = time.perf_counter()
+        while True:
+            if n_outputs_classes:
+                e = np.exp(pred - pred.max(axis=1, keepdims=True))
+                p = e / e.sum(axis=1, keepdims=True)
+                g = p.copy()
+                g[np.arange(n), y_sample.astype(np.int64)] -= 1.0
+                g *= lr
+                h = np.maximum(p * (1 - p), 1e-8)
+            else:
+                g = (pred - y_sample.reshape(-1, 1)) * lr
+                h = np.ones((n, 1))
+            leaf, feat, split, gain, hess = cv.build_tree(X_sample, g, h, max_depth=max_depth,
+                                                          split_samples=split_samples, seed=rounds, n_threads=n_threads)
+            pred += cv.predict(X_sample, [(leaf, feat, split)], k, n_threads=n_threads)
+            rounds += 1
+            dt = time.perf_counter() - t0
+            if rounds >= min_rounds and dt >= budget:
+                return rounds, dt
+
+    rounds_p, dt_p = run(cores, seconds * 0.4, 2)
+    rounds_1, dt_1 = run(1, 0.0, 1)
+    scale = n / full_rows
     return {
-        "value": rate_sample * n / full_rows,
+        "value": rounds_p / dt_p * scale,
         "unit": "rounds/s",
         "cores": cores,
         "kind": "port",
-        "sample": "first %d of %d rows, %d rounds in %.1f s on %d threads (%.3f rounds/s on the sample, "
-                  "scaled by rows)" % (n, full_rows, rounds, dt, cores, rate_sample),
+        "sample": ("all %d rows" % n if n == full_rows else "first %d of %d rows" % (n, full_rows))
+                  + "; %d threads: %d rounds in %.1f s; 1 thread: %d round(s) in %.1f s" % (cores, rounds_p, dt_p, rounds_1, dt_1)
+                  + ("" if n == full_rows else "; both scaled to the full rows by %d/%d (a round's work is linear in "
+                                               "the rows)" % (n, full_rows)),
+        "single_thread": {"value": rounds_1 / dt_1 * scale, "unit": "rounds/s", "cores": 1},
+        "host_cpu_count": os.cpu_count(),
     }
+
+
+def source_tag():
+    """Identifies the kernels a profile was taken on: the first 12 hex digits of the SHA-256 of lbt_histogram.hip."""
+    import hashlib
+
+    path = os.path.join(ROOT, "legate-boost_amd", "csrc", "lbt_histogram.hip")
+    return hashlib.sha256(open(path, "rb").read()).hexdigest()[:12]
 
 
 def measured_traffic(workload, rows, features):
     """HBM bytes per launch from rocprofv3 counter runs of this command, kept as text under profiles/.
 
-    Lines of the form `<kernel> traffic_bytes_per_launch=<number> workload=<name> rows=<n> features=<f>`;
-    only those taken on the same workload apply. Returns {} when none do."""
+    Lines of the form `<kernel> traffic_bytes_per_launch=<number> workload=<name> rows=<n> features=<f>
+    source=<tag>`; only those taken on the same workload and on the kernel source as it is now apply
+    (a counter run cannot be made from inside this program). Returns {} when none do."""
     out = {}
     path = os.path.join(ROOT, "profiles", "hbm_traffic_%s.txt" % workload)
     if not os.path.exists(path):
         return out
+    tag = source_tag()
     for line in open(path):
         parts = line.split()
         if len(parts) < 2 or "traffic_bytes_per_launch=" not in line:
             continue
         kv = dict(p.split("=", 1) for p in parts[1:] if "=" in p)
-        if kv.get("workload") == workload and int(kv.get("rows", -1)) == rows and int(kv.get("features", -1)) == features:
+        if (kv.get("workload") == workload and int(kv.get("rows", -1)) == rows
+                and int(kv.get("features", -1)) == features and kv.get("source") == tag):
             out[parts[0]] = float(kv["traffic_bytes_per_launch"])
     return out
 
@@ -143,10 +162,11 @@ def bench_training(args):
         yc = y.reshape(-1, 1)
 
     gh = (torch.empty_like(pred), torch.empty_like(pred))
+    sums = torch.empty((2, int(_lib.lib.lbt_abs_sum_chunks(n, k))), dtype=torch.float64, device=X.device)
 
-    def one_round():
+    def one_round(reference_flow=args.reference_flow):
         seed = int(rs.randint(0, 2**31))
-        if args.reference_flow:
+        if reference_flow:
             # the caller's steps as separate array operations and a traversal of X per round
             if n_classes:
                 p = torch.softmax(pred, dim=1)
@@ -160,11 +180,13 @@ def bench_training(args):
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
             pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
         else:
-            # gradient step in one pass; the prediction update takes the rows' leaves from the
-            # build: same values as PredictTask on the training rows (checked bit for bit in the tests)
-            g, h = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc, pred,
-                                         None, lr, out=gh)
-            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True, wait=False)
+            # gradient step in one pass, which also leaves the first level of the quantiser's absolute
+            # sums; the prediction update takes the rows' leaves from the build: same values as
+            # PredictTask on the training rows (checked bit for bit in the tests)
+            g, h, part = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc,
+                                               pred, None, lr, out=gh, sums=sums)
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True, wait=False,
+                               abs_sum_chunks=part)
             ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         return r
 
@@ -195,6 +217,17 @@ def bench_training(args):
     torch.cuda.synchronize()
     _lib.profile_enable(0)
     prof_all = _lib.profile_get()
+    # the other flow of a round, in the same run and on the same model: the reference loop's own
+    # steps (gradient as separate array operations, BuildTreeTask, PredictTask of the new tree)
+    # when the timed rounds took the fused steps, and the other way round
+    other_steps = max(2, min(args.steps, 5))
+    one_round(not args.reference_flow)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(other_steps):
+        one_round(not args.reference_flow)
+    torch.cuda.synchronize()
+    other_rate = other_steps / (time.perf_counter() - t0)
 
     hist, binning = prof["histogram"], prof["binning"]
     elem = X.element_size()
@@ -209,6 +242,7 @@ def bench_training(args):
     # per output (gradients are quantised once per tree, 8 bytes per pair), every row of the
     # level's nodes its (node, row) pair, every built histogram is written once.
     stage_bytes = 0.0
+    pair_extra = 0.0
     levels = []
     for d, lv in enumerate(prof["levels"]):
         # the library's own figure prices a feature value at its cached width; what is left of it
@@ -217,6 +251,7 @@ def bench_training(args):
         written = max(0.0, lv["bytes"] - own_extra - lv["built_instances"] * (f * bin_bytes + k * 8.0 + 8.0))
         ref_bytes = lv["built_instances"] * (f * elem + k * 8.0) + lv["instances"] * 8.0 + written
         stage_bytes += ref_bytes
+        pair_extra += lv["built_instances"] * k * 8.0
         levels.append({"level": d, "ms": lv["ms"] / steps, "built_rows": lv["built_instances"] / steps,
                        "built_nodes": lv["built_nodes"] / steps,
                        "GB_cached_bins": lv["bytes"] / steps / 1e9, "GBps_cached_bins": gbps(lv["bytes"], lv["ms"]),
@@ -245,6 +280,11 @@ def bench_training(args):
             "rows": n, "features": f, "outputs": k, "max_depth": depth, "split_samples": S,
             "loss_before": loss0, "loss_after": loss1,
             "prediction_update": "PredictTask" if args.reference_flow else "row->leaf map from BuildTreeTask",
+            # a round as the reference loop runs it (legateboost.py:254-275): gradient arithmetic as
+            # array operations, BuildTreeTask, PredictTask of the new tree; measured in this run
+            "reference_flow_rounds_per_s": args.steps / dt if args.reference_flow else other_rate,
+            "fused_flow_rounds_per_s": other_rate if args.reference_flow else args.steps / dt,
+            "other_flow_steps": other_steps,
         },
         # the kernel with the largest share of a round: the histogram kernel on cached bins,
         # priced on the bytes of its own input format (one or two bytes per feature value)
@@ -255,6 +295,14 @@ def bench_training(args):
             "unit": "GB/s",
             "frac": hist_achieved / HBM_PEAK_GBS,
             "traffic": traffic.get("binned_histogram_kernel"),
+            "traffic_source": "profiles/hbm_traffic_%s.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE), applies when its "
+                              "source tag equals %s" % (name, source_tag()),
+            # the histogram stage of a tree (binning pass + every histogram launch) against the bytes
+            # the reference's histogram kernel has to move for the same levels, with the quantised
+            # gradient pair of a row and output priced at 8 bytes (rounded once per tree here) and
+            # at the 16 bytes of the two doubles the reference kernel reads
+            "frac_reference_accounting": gbps(stage_bytes, stage_ms) / HBM_PEAK_GBS,
+            "frac_reference_accounting_pairs_at_16_bytes": gbps(stage_bytes + pair_extra, stage_ms) / HBM_PEAK_GBS,
             "kernel": "binned_histogram_kernel",
             "launches": hist["launches"],
             "avg_launch_ms": hist["ms"] / max(1, hist["launches"]),
@@ -281,7 +329,8 @@ def bench_training(args):
         "kernel_ms_per_round": {c: prof_all[c]["ms"] / 2 for c in _lib.PROF_CLASSES},
     }
     if not args.no_cpu_baseline:
-        ns = min(n, 500_000 if cfg != 1 else n)
+        # config 2 (the headline) on all of its rows; the wider configurations on a row sample
+        ns = n if cfg <= 2 else min(n, 500_000)
         out["cpu_baseline"] = cpu_baseline_build(X[:ns].cpu().numpy(), y[:ns].cpu().numpy(), depth, S, lr, n,
                                                  args.cpu_seconds, n_classes)
     return out

@@ -66,6 +66,12 @@ typedef struct lbt_build_params {
   double l2_regularization;
   double min_split_gain;
   int64_t hist_cache_bytes;
+  /* Optional, device: the first level of the sums of |g| and |h| as lbt_weighted_gradient_sums
+   * writes them for exactly these g and h ([2][lbt_abs_sum_chunks(n_rows, n_outputs)] doubles).
+   * With it the build skips its own first pass over g and h for the quantiser's scale
+   * (build_tree.cu:77-83); the scale, and with it every result, is the same bit for bit.
+   * NULL: the build sums g and h itself. Sums that belong to other gradients give a wrong scale. */
+  const double* abs_sum_chunks;
 } lbt_build_params;
 
 /* Optional observation points of lbt_build_tree, for parity tests and
@@ -306,6 +312,21 @@ int lbt_update_tree(void* stream, const void* X, int32_t x_dtype, int64_t n_rows
 int lbt_weighted_gradient(void* stream, int32_t objective, const double* pred, const double* y,
                           const double* sample_weight, double learning_rate, int64_t n_rows,
                           int32_t n_outputs, double* g, double* h);
+
+/*
+ * lbt_weighted_gradient that also leaves the first level of the quantiser's two absolute sums
+ * (legateboost.py:260-275 followed by build_tree.cu:77-83): the pass that produces g and h adds
+ * up |g| and |h| per chunk of 4096 consecutive entries of the flat [n_rows * n_outputs] arrays,
+ * in the fixed order the quantiser uses, so that lbt_build_tree (lbt_build_params.abs_sum_chunks)
+ * need not read g and h once more for its scale. g and h are the same bits lbt_weighted_gradient
+ * writes.
+ *   abs_sum_chunks  device double [2][lbt_abs_sum_chunks(n_rows, n_outputs)]: the chunk sums of
+ *                   |g|, then those of |h|
+ */
+int64_t lbt_abs_sum_chunks(int64_t n_rows, int32_t n_outputs);
+int lbt_weighted_gradient_sums(void* stream, int32_t objective, const double* pred, const double* y,
+                               const double* sample_weight, double learning_rate, int64_t n_rows,
+                               int32_t n_outputs, double* g, double* h, double* abs_sum_chunks);
 
 /*
  * pred[r][k] += leaf_value[row_leaf[r]][k]: the update `train_pred += model.predict(X)` of

@@ -1346,23 +1346,34 @@ int run_split_samples(hipStream_t stream, const T* X, int64_t row_offset, int64_
 // GradientQuantiser and reduce_base_sums (build_tree.cu:51-140, :168-204): the two absolute sums
 // in a fixed order, the scales, one rounding per (row, output), and the sums of the rounded pairs
 // added to root_sums[k] (which the caller has cleared). part_a/part_b: two levels of partial sums.
+// first_level: the chunk sums of |g| and |h| if the caller has them already ([2][chunks], see
+// lbt_weighted_gradient_sums), else null.
 int run_quantiser(hipStream_t stream, const double* g, const double* h, int64_t N, int K, int64_t row_offset,
                   int32_t seed, double* const (&part_a)[2], double* const (&part_b)[2], double* scales,
-                  unsigned long long* qstats, int2* qgh, I64Pair* root_sums)
+                  unsigned long long* qstats, int2* qgh, I64Pair* root_sums, const double* first_level = nullptr)
 {
   auto blocks = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
   int64_t n = N * K;
   int64_t m = (n + 4095) / 4096;
-  abs_sum_level_kernel<true><<<static_cast<unsigned>(m), kThreads, 0, stream>>>(g, h, n, part_a[0], part_b[0]);
+  const double* in_a = part_a[0];
+  const double* in_b = part_b[0];
+  if (first_level != nullptr) {
+    in_a = first_level;
+    in_b = first_level + m;
+  } else {
+    abs_sum_level_kernel<true><<<static_cast<unsigned>(m), kThreads, 0, stream>>>(g, h, n, part_a[0], part_b[0]);
+  }
   int cur = 0;
   while (m > 1) {
     int64_t m2 = (m + 4095) / 4096;
-    abs_sum_level_kernel<false><<<static_cast<unsigned>(m2), kThreads, 0, stream>>>(part_a[cur], part_b[cur], m,
-                                                                                     part_a[cur ^ 1], part_b[cur ^ 1]);
+    abs_sum_level_kernel<false><<<static_cast<unsigned>(m2), kThreads, 0, stream>>>(in_a, in_b, m, part_a[cur ^ 1],
+                                                                                     part_b[cur ^ 1]);
     cur ^= 1;
-    m = m2;
+    in_a = part_a[cur];
+    in_b = part_b[cur];
+    m    = m2;
   }
-  scales_kernel<<<1, 64, 0, stream>>>(part_a[cur], part_b[cur], scales, qstats);
+  scales_kernel<<<1, 64, 0, stream>>>(in_a, in_b, scales, qstats);
   if (K > 1 && K <= kQuantiseFlatMaxK) {
     const unsigned gx =
       std::max<unsigned>(std::min<unsigned>(blocks(N * K, kThreads), 2048u), blocks(K, kThreads));
@@ -1410,7 +1421,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   {
     ProfScope ps(LBT_PROF_QUANTISE, stream, static_cast<double>(N) * K * (16 + 16 + 8));
     LBT_TRY(run_quantiser(stream, g, h, N, K, row_offset, prm.seed, L.part_a, L.part_b, L.scales, L.qstats, L.qgh,
-                          L.node_sums));
+                          L.node_sums, prm.abs_sum_chunks));
     root_leaf_kernel<<<blocks(K, 64), 64, 0, stream>>>(leaf, L.node_sums, K, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization);
   }

@@ -31,6 +31,7 @@ class BuildParams(C.Structure):
         ("l2_regularization", C.c_double),
         ("min_split_gain", C.c_double),
         ("hist_cache_bytes", C.c_int64),
+        ("abs_sum_chunks", C.c_void_p),
     ]
 
 
@@ -129,6 +130,11 @@ def _load():
     lib.lbt_weighted_gradient.restype = C.c_int
     lib.lbt_weighted_gradient.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
                                           C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.lbt_abs_sum_chunks.restype = C.c_int64
+    lib.lbt_abs_sum_chunks.argtypes = [C.c_int64, C.c_int32]
+    lib.lbt_weighted_gradient_sums.restype = C.c_int
+    lib.lbt_weighted_gradient_sums.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
+                                               C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.lbt_add_leaf_values.restype = C.c_int
     lib.lbt_add_leaf_values.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int32,
                                         C.c_void_p]
@@ -162,7 +168,8 @@ lib = _load()
 EXPORTS = [
     "lbt_last_error", "lbt_version", "lbt_release_thread_resources", "lbt_build_tree_workspace_bytes", "lbt_build_tree", "lbt_build_tree_async", "lbt_predict",
     "lbt_predict_workspace_bytes", "lbt_pack_ensemble", "lbt_predict_packed",
-    "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_add_leaf_values",
+    "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_weighted_gradient_sums",
+    "lbt_abs_sum_chunks", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_select_split_samples_workspace_bytes", "lbt_select_split_samples",
     "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_quantise_gradients_static", "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",

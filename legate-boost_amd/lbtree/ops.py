@@ -56,10 +56,11 @@ class BuildResult:
 
 def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0, l2_regularization=1.0,
                min_split_gain=0.0, feature_set=None, dataset_rows=None, row_offset=0, hist_cache_bytes=0,
-               taps=False, taps_levels=False, row_leaf=False, wait=True):
+               taps=False, taps_levels=False, row_leaf=False, wait=True, abs_sum_chunks=None):
     """BUILD_TREE (legateboost/models/tree.py:104-191). Returns a BuildResult with the five task
     outputs as CUDA tensors; with taps=True also the observation points. wait=False returns
-    without synchronising the stream (lbt_build_tree_async; not together with taps=True)."""
+    without synchronising the stream (lbt_build_tree_async; not together with taps=True).
+    abs_sum_chunks: the chunk sums weighted_gradient(..., sums=True) returned for these g and h."""
     X = _check_x(X)
     g = as_device(g, torch.float64)
     h = as_device(h, torch.float64)
@@ -72,6 +73,11 @@ def build_tree(X, g, h, *, max_depth, split_samples, seed, l1_regularization=0.0
     prm = _lib.BuildParams(max_depth, max_nodes, split_samples, seed,
                            dataset_rows if dataset_rows is not None else n, l1_regularization,
                            l2_regularization, min_split_gain, hist_cache_bytes)
+    if abs_sum_chunks is not None:
+        if not (abs_sum_chunks.is_cuda and abs_sum_chunks.dtype == torch.float64 and abs_sum_chunks.is_contiguous()
+                and abs_sum_chunks.numel() == 2 * _lib.lib.lbt_abs_sum_chunks(n, k)):
+            raise _lib.LbtError("abs_sum_chunks must be the [2][chunks] float64 CUDA tensor of weighted_gradient")
+        prm.abs_sum_chunks = abs_sum_chunks.data_ptr()
     nbytes = _lib.lib.lbt_build_tree_workspace_bytes(n, f, k, max_depth, split_samples, _DT[X.dtype], hist_cache_bytes)
     if nbytes == 0:
         # let the library produce the message for the offending argument
@@ -251,10 +257,12 @@ def update_tree(X, g, h, feature, split_value, l1_regularization, l2_regularizat
 _OBJECTIVES = {"squared_error": _lib.LBT_OBJ_SQUARED_ERROR, "log_loss": _lib.LBT_OBJ_LOG_LOSS}
 
 
-def weighted_gradient(objective, y, pred, sample_weight=None, learning_rate=1.0, out=None):
+def weighted_gradient(objective, y, pred, sample_weight=None, learning_rate=1.0, out=None, sums=False):
     """LBBase._get_weighted_gradient (legateboost/legateboost.py:189-224) for "squared_error" or
     "log_loss" in one pass. pred: raw predictions [n, K]; y: [n, K], or [n] / [n, 1] class labels
-    for log loss with K > 1. Returns (g, h); `out=(g, h)` reuses two buffers of pred's shape."""
+    for log loss with K > 1. Returns (g, h); `out=(g, h)` reuses two buffers of pred's shape.
+    sums=True (or a [2][chunks] float64 tensor to fill): also the chunk sums of |g| and |h| that
+    build_tree(abs_sum_chunks=...) takes in place of its own pass over g and h; returns (g, h, sums)."""
     pred = as_device(pred, torch.float64)
     y = as_device(y, torch.float64)
     if pred.dim() != 2:
@@ -271,6 +279,16 @@ def weighted_gradient(objective, y, pred, sample_weight=None, learning_rate=1.0,
     if objective not in _OBJECTIVES:
         raise _lib.LbtError("unknown objective %r" % (objective,))
     g, h = out if out is not None else (torch.empty_like(pred), torch.empty_like(pred))
+    if sums is not False and sums is not None:
+        m = int(_lib.lib.lbt_abs_sum_chunks(n, k))
+        part = sums if isinstance(sums, torch.Tensor) else torch.empty((2, m), dtype=torch.float64, device=pred.device)
+        if part.numel() != 2 * m or part.dtype != torch.float64 or not part.is_cuda:
+            raise _lib.LbtError("sums must be a float64 CUDA tensor of 2 x %d entries" % m)
+        rc = _lib.lib.lbt_weighted_gradient_sums(_stream(), _OBJECTIVES[objective], pred.data_ptr(), y.data_ptr(),
+                                                 w.data_ptr() if w is not None else None, float(learning_rate), n, k,
+                                                 g.data_ptr(), h.data_ptr(), part.data_ptr())
+        _lib.check(rc)
+        return g, h, part
     rc = _lib.lib.lbt_weighted_gradient(_stream(), _OBJECTIVES[objective], pred.data_ptr(), y.data_ptr(),
                                         w.data_ptr() if w is not None else None, float(learning_rate), n, k,
                                         g.data_ptr(), h.data_ptr())

@@ -368,6 +368,52 @@ def test_log_loss_gradient_matches_oracle(k):
     assert np.isfinite(gu.cpu(g_g)).all() and (gu.cpu(h_g) >= 1e-8).all()
 
 
+@pytest.mark.parametrize("objective,n,k", [("squared_error", 100003, 1), ("squared_error", 20481, 3),
+                                           ("log_loss", 70001, 1), ("log_loss", 30011, 8), ("log_loss", 9001, 5),
+                                           ("log_loss", 300, 13)])
+def test_gradient_pass_with_the_quantisers_sums(objective, n, k):
+    """lbt_weighted_gradient_sums writes the same g and h as lbt_weighted_gradient and the first level
+    of the quantiser's absolute sums; a build that is handed those sums skips its own pass over g
+    and h and must give the oracle's scales, rounded pairs and tree bit for bit."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    rs = np.random.RandomState(n + k)
+    pred = 3 * rs.normal(size=(n, k))
+    if objective == "squared_error":
+        y = rs.normal(size=(n, k))
+    else:
+        y = rs.randint(0, max(k, 2), n).astype(np.float64)
+        y = y.reshape(-1, 1) if k == 1 else y
+    w = rs.gamma(2.0, size=n)
+    g0, h0 = ops.weighted_gradient(objective, y, pred, w, 0.3)
+    g1, h1, sums = ops.weighted_gradient(objective, y, pred, w, 0.3, sums=True)
+    assert torch.equal(g0, g1) and torch.equal(h0, h1)
+    # the chunk sums against a plain numpy restatement of the fixed order: 4096 entries per chunk,
+    # lane t adds entries t, t + 256, ..., then a binary tree over the 256 lanes
+    for arr, got in ((gu.cpu(g1), gu.cpu(sums[0])), (gu.cpu(h1), gu.cpu(sums[1]))):
+        flat = np.abs(arr.reshape(-1))
+        m = (flat.size + 4095) // 4096
+        padded = np.zeros(m * 4096)
+        padded[: flat.size] = flat
+        lanes = np.zeros((m, 256))
+        for j in range(16):
+            lanes += padded.reshape(m, 16, 256)[:, j, :]
+        stride = 128
+        while stride >= 1:
+            lanes[:, :stride] += lanes[:, stride: 2 * stride]
+            stride //= 2
+        assert np.array_equal(got, lanes[:, 0])
+    X = rs.normal(size=(n, 6)).astype(np.float32)
+    cr = orc.build_tree(X, gu.cpu(g1), gu.cpu(h1), max_depth=4, split_samples=32, seed=11)
+    gr = ops.build_tree(X, g1, h1, max_depth=4, split_samples=32, seed=11, taps=True, abs_sum_chunks=sums)
+    gu.assert_tree_parity(gr, cr)
+    # the asynchronous form, as the boosting loop calls it
+    r2 = ops.build_tree(X, g1, h1, max_depth=4, split_samples=32, seed=11, wait=False, abs_sum_chunks=sums)
+    assert torch.equal(r2.leaf_value, gr.leaf_value) and torch.equal(r2.feature, gr.feature)
+
+
 # depth 13 / 14: the last level has 4096 / 8192 segments, either side of what the windowed leaf
 # kernel indexes; 600 split samples: two-byte bins; depth 1: no bin cache
 @pytest.mark.parametrize("k,depth,s", [(1, 6, 64), (4, 6, 64), (1, 13, 16), (1, 14, 16), (2, 5, 600), (1, 1, 64)])
