@@ -538,6 +538,159 @@ __global__ void __launch_bounds__(kThreads)
   if (threadIdx.x == 0) partial[static_cast<int64_t>(blockIdx.x) * n_chunks + blockIdx.y] = best;
 }
 
+// Scan, sibling subtraction and split evaluation in one pass over the histograms
+// (build_tree.cu:597-668 and :682-740): one wave per (built node, feature) takes 64 bins of the
+// feature at a time and, output by output, forms the running sums, stores them under the
+// reference's rule, derives the sibling's bins where the sibling is not built, and adds the
+// output's share to the gain of every bin of the node and of the sibling while the sums are
+// still in registers. The histograms are read once instead of twice, and the candidates of a
+// node come out per feature (split_apply_kernel reduces them with the same total order).
+// Where the reference's scan returns early for an output (node sum of hessians not positive,
+// :613) the bins of that output stay as they are in memory, for the node and for its sibling,
+// and the gains are formed from those values, as the reference's split kernel would read them.
+constexpr int kFusedMaxK   = 64;  // lane k of the wave keeps the running sums of output k
+
+__device__ inline void add_gain(double& gain, bool& dead, const I64Pair& ls, const I64Pair& ns, double inv_g,
+                                double inv_h, double l1, double reg, double min_split_gain)
+{
+  const int64_t rg = ns.grad - ls.grad, rh = ns.hess - ls.hess;
+  if (dead) return;
+  if (ls.hess <= 0 || rh <= 0) {
+    // build_tree.cu:727-730: one output without a valid split on this bin voids the bin
+    dead = true;
+    gain = 0;
+    return;
+  }
+  gain += calculate_gain(static_cast<double>(ls.grad) * inv_g, static_cast<double>(ls.hess) * inv_h,
+                         static_cast<double>(rg) * inv_g, static_cast<double>(rh) * inv_h,
+                         static_cast<double>(ns.grad) * inv_g, static_cast<double>(ns.hess) * inv_h, l1, reg,
+                         min_split_gain);
+}
+
+__device__ inline Cand wave_best(Cand c)
+{
+  for (int off = 32; off >= 1; off >>= 1) {
+    Cand o;
+    o.gain = __shfl_down(c.gain, off, 64);
+    o.bin  = __shfl_down(c.bin, off, 64);
+    if (cand_better(o, c)) c = o;
+  }
+  return c;  // valid on lane 0
+}
+
+__global__ void __launch_bounds__(kThreads)
+  scan_split_kernel(HistView hist, const I64Pair* node_sums, int F, const int32_t* row_pointers, int node_begin,
+                    int n_nodes, const uint8_t* feature_set, const double* scales, double l1, double l2,
+                    double min_split_gain, Cand* partial)
+{
+  const int lane     = threadIdx.x & 63;
+  const int64_t rank = (blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x) >> 6;
+  const int i        = static_cast<int>(rank / n_nodes);
+  const int j        = static_cast<int>(rank % n_nodes);
+  if (i >= F) return;
+  const int K      = hist.K;
+  const int node   = node_begin + j;
+  const int parent = parent_of(node);
+  if (!compute_histogram_bin(node, node_sums, K, hist.contains(parent))) return;
+  const int sib     = node == 0 ? -1 : sibling_of(node);
+  const bool derive = node != 0 && !compute_histogram_bin(sib, node_sums, K, hist.contains(parent));
+  // which of the two are split candidates at all (build_tree.cu:712), and on this feature
+  const bool usable   = feature_set == nullptr || feature_set[i] != 0;
+  const bool eval_n   = usable && node_sums[static_cast<int64_t>(node) * K].hess > 0;
+  const bool eval_s   = usable && derive && node_sums[static_cast<int64_t>(sib) * K].hess > 0;
+  const double inv_g = scales[2], inv_h = scales[3];
+  const double reg   = 1e-5 > l2 ? 1e-5 : l2;
+  // Nothing to scan (no output of the node has a positive sum of hessians: an empty node, as
+  // most nodes of a deep level are) and nothing to evaluate: the bins stay as they are.
+  bool any_scan = false;
+  for (int k = 0; k < K; k++) any_scan |= node_sums[static_cast<int64_t>(node) * K + k].hess > 0;
+  if (!any_scan && !eval_n && !eval_s) {
+    if (lane == 0) {
+      partial[static_cast<int64_t>(j) * F + i] = Cand{0.0, -1};
+      if (derive) partial[static_cast<int64_t>(sib - node_begin) * F + i] = Cand{0.0, -1};
+    }
+    return;
+  }
+  int64_t agg_g = 0, agg_h = 0;  // lane k: sums of output k over the tiles done so far
+  const int fb = row_pointers[i], fe = row_pointers[i + 1];
+  Cand best_n{0.0, -1}, best_s{0.0, -1};
+  // The bins of the next (tile, output) and the parent's are requested before the current ones
+  // are scanned and stored: the stores would otherwise keep every load behind them, and a wave
+  // would wait for memory once per tile and output.
+  auto fetch = [&](int base, int k, I64Pair& ns, I64Pair& val, I64Pair& other) {
+    const int b = base + lane;
+    ns          = node_sums[static_cast<int64_t>(node) * K + k];
+    val = other = I64Pair{0, 0};
+    if (b < fe) {
+      val = *hist.at(node, k, b);  // what the split evaluation reads for this bin
+      // the parent's bin where the sibling is derived from it, else the sibling's bin as it is in memory
+      if (derive) other = ns.hess > 0 ? *hist.at(parent, k, b) : *hist.at(sib, k, b);
+    }
+  };
+  I64Pair ns_next, val_next, other_next;
+  if (fb < fe) fetch(fb, 0, ns_next, val_next, other_next);
+  for (int base = fb; base < fe; base += 64) {
+    const int bin = base + lane;
+    const bool in = bin < fe;
+    double gain_n = 0.0, gain_s = 0.0;
+    bool dead_n = false, dead_s = false;
+    for (int k = 0; k < K; k++) {
+      const I64Pair ns = ns_next;
+      I64Pair val = val_next, sval = other_next;
+      if (k + 1 < K)
+        fetch(base, k + 1, ns_next, val_next, other_next);
+      else if (base + 64 < fe)
+        fetch(base + 64, 0, ns_next, val_next, other_next);
+      if (ns.hess > 0) {
+        int64_t eg = val.grad, eh = val.hess;
+        for (int off = 1; off < 64; off <<= 1) {
+          const int64_t og = __shfl_up(eg, off, 64);
+          const int64_t oh = __shfl_up(eh, off, 64);
+          if (lane >= off) {
+            eg += og;
+            eh += oh;
+          }
+        }
+        const int64_t tile_g = __shfl(eg, 63, 64), tile_h = __shfl(eh, 63, 64);
+        eg += __shfl(agg_g, k, 64);
+        eh += __shfl(agg_h, k, 64);
+        // the reference skips the store when the running sum is not positive
+        // (build_tree.cu:645); the raw bin value then stays in place
+        if (in && (eg > 0 || eh > 0)) {
+          val                    = I64Pair{eg, eh};
+          *hist.at(node, k, bin) = val;
+        }
+        if (lane == k) {
+          agg_g += tile_g;
+          agg_h += tile_h;
+        }
+        if (derive && in) {
+          sval                  = I64Pair{sval.grad - val.grad, sval.hess - val.hess};
+          *hist.at(sib, k, bin) = sval;
+        }
+      }
+      if (eval_n && in) add_gain(gain_n, dead_n, val, ns, inv_g, inv_h, l1, reg, min_split_gain);
+      if (eval_s && in)
+        add_gain(gain_s, dead_s, sval, node_sums[static_cast<int64_t>(sib) * K + k], inv_g, inv_h, l1, reg,
+                 min_split_gain);
+    }
+    if (in && gain_n > 0) {
+      const Cand c{gain_n, bin};
+      if (cand_better(c, best_n)) best_n = c;
+    }
+    if (in && gain_s > 0) {
+      const Cand c{gain_s, bin};
+      if (cand_better(c, best_s)) best_s = c;
+    }
+  }
+  best_n = wave_best(best_n);
+  if (lane == 0) partial[static_cast<int64_t>(j) * F + i] = best_n;
+  if (derive) {
+    best_s = wave_best(best_s);
+    if (lane == 0) partial[static_cast<int64_t>(sib - node_begin) * F + i] = best_s;
+  }
+}
+
 __global__ void __launch_bounds__(64)
   split_apply_kernel(HistView hist, I64Pair* node_sums, const int32_t* bin_feature,
                      const double* proposals_as_double, const double* scales, double l1, double l2,
@@ -1276,7 +1429,8 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
   L.partial_list_count = ar.take<int32_t>(kPartialMaxLists);
   L.partial_count = ar.take<int32_t>(1);
   L.level_totals  = ar.take<LevelMeta>(max_depth > 0 ? max_depth : 1);
-  const int64_t max_chunks = (static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk;
+  // candidates per node: one per chunk of bins (split_eval_kernel) or one per feature (scan_split_kernel)
+  const int64_t max_chunks = std::max<int64_t>((static_cast<int64_t>(F) * S + kSplitChunk - 1) / kSplitChunk, F);
   L.partial       = ar.take<Cand>(level_nodes * max_chunks);
   L.hist_bytes    = hist_bytes_bound(F, K, S, max_depth, cache_bytes);
   L.hist          = reinterpret_cast<I64Pair*>(ar.take<char>(L.hist_bytes));
@@ -1548,21 +1702,36 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
         hb.level_total = L.level_totals + depth; hb.n_rows = N;
         LBT_TRY(hist_launch(stream, hs, hb, depth));
       }
-      {
+      // One pass that scans and evaluates reads the histograms once instead of twice and saves a
+      // launch per level. With a single output and many nodes (the deep levels of a deep tree,
+      // most of whose nodes are empty or small) the two kernels are faster: the evaluation then
+      // runs over all bins of a node side by side, not feature by feature behind the scan.
+      const bool fused = K <= kFusedMaxK && (K >= 2 || n_nodes <= 256);
+      if (fused) {
         ProfScope ps(LBT_PROF_SCAN, stream);
-        int64_t waves = static_cast<int64_t>(F) * n_nodes;
-        dim3 grid(blocks(waves, kThreads / 64), K);
-        scan_kernel<<<grid, kThreads, 0, stream>>>(hv, L.node_sums, F, L.row_pointers, batch_begin, n_nodes);
-      }
-      {
+        const int64_t waves = static_cast<int64_t>(F) * n_nodes;
+        scan_split_kernel<<<blocks(waves, kThreads / 64), kThreads, 0, stream>>>(
+          hv, L.node_sums, F, L.row_pointers, batch_begin, n_nodes, feature_set, L.scales, prm.l1_regularization,
+          prm.l2_regularization, prm.min_split_gain, L.partial);
+      } else {
+        {
+          ProfScope ps(LBT_PROF_SCAN, stream);
+          int64_t waves = static_cast<int64_t>(F) * n_nodes;
+          dim3 grid(blocks(waves, kThreads / 64), K);
+          scan_kernel<<<grid, kThreads, 0, stream>>>(hv, L.node_sums, F, L.row_pointers, batch_begin, n_nodes);
+        }
         ProfScope ps(LBT_PROF_SPLIT, stream);
         dim3 grid(n_nodes, n_chunks);
         split_eval_kernel<<<grid, kThreads, 0, stream>>>(hv, L.node_sums, L.bin_feature, feature_set, L.scales,
                                                          prm.l1_regularization, prm.l2_regularization,
                                                          prm.min_split_gain, batch_begin, n_chunks, L.partial);
+      }
+      {
+        ProfScope ps(LBT_PROF_SPLIT, stream);
+        const int n_cands = fused ? F : n_chunks;
         split_apply_kernel<<<n_nodes, 64, 0, stream>>>(hv, L.node_sums, L.bin_feature, L.proposals_d, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization, batch_begin,
-                                                       n_chunks, L.partial, leaf, feature, split, gain, L.row_pointers,
+                                                       n_cands, L.partial, leaf, feature, split, gain, L.row_pointers,
                                                        L.split_bin);
       }
     }

@@ -1294,13 +1294,20 @@ __global__ void __launch_bounds__(kHistThreads)
       }
     }
     if constexpr (kRoot) {
-      // feature-major copy (one output's workgroups do it); rows past the end of the tile hold
-      // the bins of the tile's first row, and bins_t is padded to whole groups of rows
-      if (k == 0 && (valid_c & 1u)) {
+      // feature-major copy; rows past the end of the tile hold the bins of the tile's first row,
+      // and bins_t is padded to whole groups of rows
+      // the workgroups of the K outputs read the same records: they share the copy between them,
+      // output k takes every K-th piece of four features (one output's workgroups alone would
+      // write K times as long as the others and hold the launch up)
+      if (valid_c & 1u) {
         const int64_t row0 = row_c[0];
         if constexpr (BV == 16) {
           BinT* dst = bins_t + static_cast<int64_t>(f0 + fl) * bins_t_stride + row0;
           auto put  = [&](int i, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+            if ((lr * 4 + i) % a.K != k) {
+              dst += 4 * bins_t_stride;
+              return;
+            }
             uint32_t o[4];
             turn_bytes(w0, w1, w2, w3, o);
 #pragma unroll
@@ -1324,7 +1331,7 @@ __global__ void __launch_bounds__(kHistThreads)
           o[3] = make_uint2((hi[0] >> 16) | (hi[1] & 0xffff0000u), (hi[2] >> 16) | (hi[3] & 0xffff0000u));
 #pragma unroll
           for (int v = 0; v < 4; v++)
-            if (fl + v < gs)
+            if (fl + v < gs && (lr * 4 + v) % a.K == k)
               *reinterpret_cast<uint2*>(bins_t + static_cast<int64_t>(f0 + fl + v) * bins_t_stride + row0) = o[v];
         }
       }

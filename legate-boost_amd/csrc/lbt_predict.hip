@@ -113,7 +113,7 @@ struct PackedNode;
 template <>
 struct alignas(8) PackedNode<float> {
   float thr;
-  uint32_t feat_right;  // feature in the low half, right child in the high half
+  uint32_t feat_right;  // byte offset of the feature in a row (4 * feature) in the low half, right child in the high half
 };
 template <>
 struct alignas(16) PackedNode<double> {
@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(256)
   const int right = is_leaf ? i : 2 * i + 2;
   if constexpr (sizeof(T) == 4) {
     nd.thr        = is_leaf ? __uint_as_float(0x7fc00000u) : round_down_to_float(tr.split[i]);
-    nd.feat_right = (is_leaf ? 0u : static_cast<uint32_t>(ft)) | (static_cast<uint32_t>(right) << 16);
+    nd.feat_right = (is_leaf ? 0u : static_cast<uint32_t>(ft) * 4u) | (static_cast<uint32_t>(right) << 16);
   } else {
     nd.thr   = is_leaf ? __longlong_as_double(0x7ff8000000000000LL) : tr.split[i];
     nd.feat  = is_leaf ? 0 : ft;
@@ -290,10 +290,22 @@ __device__ __forceinline__ void add_in_order_from(double& acc, const double (&va
     add_in_order_from<S, jj + 1>(acc, val, cnt);
   }
 }
+template <typename S, int jj>
+__device__ __forceinline__ void add_all_in_order_from(double& acc, const double (&val)[S::kLaneTrees])
+{
+  if constexpr (jj < S::kBatchTrees) {
+    acc += from_owner<S, jj>(val);
+    add_all_in_order_from<S, jj + 1>(acc, val);
+  }
+}
 template <typename S>
 __device__ __forceinline__ void add_in_order(double& acc, const double (&val)[S::kLaneTrees], int cnt)
 {
-  add_in_order_from<S, 0>(acc, val, cnt);
+  // all batches but the last are full: no test per tree then
+  if (cnt == S::kBatchTrees)
+    add_all_in_order_from<S, 0>(acc, val);
+  else
+    add_in_order_from<S, 0>(acc, val, cnt);
 }
 template <typename S, int kAcc, int jj>
 __device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
@@ -402,7 +414,8 @@ __global__ void __launch_bounds__(kTileThreads)
       for (int j = 0; j < kLaneTrees; j++) {
         const PackedNode<T> nd = s_nodes[base[j] + pos[j]];
         if constexpr (sizeof(T) == 4) {
-          const float xv = my_x[nd.feat_right & 0xffffu];
+          const float xv = *reinterpret_cast<const float*>(reinterpret_cast<const unsigned char*>(my_x) +
+                                                           (nd.feat_right & 0xffffu));
           pos[j]         = static_cast<int>(nd.feat_right >> 16) - (xv <= nd.thr ? 1 : 0);
         } else {
           const double xv = my_x[nd.feat];
@@ -487,7 +500,7 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
                lbt_packed_ensemble* ens)
 {
   *ens = lbt_packed_ensemble{};
-  if (buffer == nullptr || K > kTileMaxK || F > 65535) return LBT_OK;
+  if (buffer == nullptr || K > kTileMaxK || F > 16383) return LBT_OK;  // a float node holds 4 * feature in 16 bits
   int64_t total_nodes = 0;
   int max_nodes       = 0;
   for (int i = 0; i < n_trees; i++) {
@@ -811,7 +824,7 @@ int lbt_pack_ensemble(void* stream, int32_t x_dtype, int32_t n_features, int32_t
     LBT_TRY(lbt::pack_tiled<double>(s, n_features, n_trees, leaf, feature, split, tree_nodes, n_outputs, buffer,
                                     buffer_bytes, ensemble));
   if (ensemble->data == nullptr) {
-    lbt::set_error("ensemble does not fit the packed form (more than %d outputs, more than 65535 features or "
+    lbt::set_error("ensemble does not fit the packed form (more than %d outputs, more than 16383 features or "
                    "nodes per tree, or rows too wide for the LDS): use lbt_predict", lbt::kTileMaxK);
     return LBT_ERR_UNSUPPORTED;
   }
