@@ -416,15 +416,16 @@ struct Stripes {
 // histogram starts from zero and the parked parts of a node are added after the launch): the
 // sums are stored as they are, which neither waits for a load nor occupies the L2's atomic units.
 __device__ inline void merge_striped(unsigned long long* s_hist, const Stripes& st, const int* s_off, I64Pair* dst,
-                                     bool sole_owner)
+                                     bool sole_owner, int gs)
 {
   const int words = st.words();
   for (int i = threadIdx.x; i < words; i += kHistThreads) {
     const unsigned long long v = s_hist[i];
-    if (v != 0) {
+    const int col              = i & ((1 << st.log_w) - 1);
+    if (v != 0 && col < gs) {  // columns past the group's features collect the adds of record padding
       int32_t gv, hv;
       unpack_pair(v, gv, hv);
-      I64Pair* d = dst + s_off[i & ((1 << st.log_w) - 1)] + (i >> st.log_w);
+      I64Pair* d = dst + s_off[col] + (i >> st.log_w);
       if (sole_owner) {
         *d = I64Pair{gv, hv};
       } else {
@@ -452,10 +453,11 @@ struct PartialSink {
 // clears them; a pass after the launch adds up the slots of every (node, group, output) with
 // plain loads. Without a free slot the atomics do it. All threads of the workgroup call this.
 __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I64Pair* dst, const PartialSink& sink,
-                                          int tag, int* s_slot, bool sole_owner, const Stripes& st, const int* s_off)
+                                          int tag, int* s_slot, bool sole_owner, const Stripes& st, const int* s_off,
+                                          int gs)
 {
   if (sole_owner && st.log_w >= 0) {
-    merge_striped(s_hist, st, s_off, dst, true);
+    merge_striped(s_hist, st, s_off, dst, true, gs);
     return;
   }
   if (sole_owner) {
@@ -499,7 +501,7 @@ __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I6
       s_hist[i] = 0;
     }
   } else if (st.log_w >= 0) {
-    merge_striped(s_hist, st, s_off, dst, false);
+    merge_striped(s_hist, st, s_off, dst, false, gs);
   } else {
     merge_sub_histogram(s_hist, nb, dst);
   }
@@ -1274,7 +1276,7 @@ __global__ void __launch_bounds__(kHistThreads)
         if (cur_node >= 0)
           park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink,
                              (cur_node - w.level_first - w.j0) * w.n_gk + gk, &s_slot,
-                             owners && tc.node != cur_node && node_rows == node_total, st, s_off);
+                             owners && tc.node != cur_node && node_rows == node_total, st, s_off, gs);
         __syncthreads();
         if (tc.node != cur_node) {
           node_rows  = 0;
@@ -1353,8 +1355,10 @@ __global__ void __launch_bounds__(kHistThreads)
           // the lanes that take part in it
           for (int v = 0; v < BV; v++) {
             if constexpr (kStriped) {
-              if (has & (1u << v))
-                atomicAdd(reinterpret_cast<unsigned long long*>(smem_raw + ((rel[v] << stripe_shift) + c_base[v])), packed);
+              // no test per bin: the bytes past the group's last feature are zeros and belong to columns of
+              // the array that no feature owns and no merge reads (an atomic costs by the instruction, not
+              // by the lanes that take part, and a test costs two branches)
+              atomicAdd(reinterpret_cast<unsigned long long*>(smem_raw + ((rel[v] << stripe_shift) + c_base[v])), packed);
             } else {
               if (v < nv) atomicAdd(&s_hist[c_base[v] + rel[v]], packed);
             }
@@ -1402,7 +1406,7 @@ __global__ void __launch_bounds__(kHistThreads)
   __syncthreads();
   if (cur_node >= 0)
     park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink, (cur_node - w.level_first - w.j0) * w.n_gk + gk,
-                       &s_slot, owners && node_rows == node_total, st, s_off);
+                       &s_slot, owners && node_rows == node_total, st, s_off, gs);
 }
 
 template <typename T, int VEC, bool kIdentityRows>
@@ -1458,8 +1462,12 @@ int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& 
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
     // meeting points only between workgroups that run at the same time: one that waits for a
-    // workgroup not yet started would sit out its whole wait at every meeting point
-    kRoot && a.w.n_gk > 1 && a.w.all_resident && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr, sink);
+    // workgroup not yet started would sit out its whole wait at every meeting point. And only for
+    // single-output trees, whose root launch is bound by the memory traffic the meetings save; with
+    // several outputs the records are found in the L2 anyway (the workgroups of the other outputs
+    // asked for them) and the waiting is all that is left (2M x 200, 8 outputs: 1.27 ms with, 0.95 ms without)
+    kRoot && a.K == 1 && a.w.n_gk > 1 && a.w.all_resident && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr,
+    sink);
   return LBT_OK;
 }
 template <typename BinT, int BV, bool kEmbed>
