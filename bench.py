@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--reference-flow", action="store_true",
                     help="update the training predictions with a PredictTask per round (as the reference loop does) instead of the row->leaf map that BuildTreeTask can return")
+    ap.add_argument("--hist-cache-bytes", type=int, default=0,
+                    help="bytes of histograms BuildTreeTask keeps (0 = the reference's 1e9, build_tree.cu:1004); a larger "
+                         "cache builds the same trees and lets deeper levels derive siblings by subtraction")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 4 GiB device copy five times (to scale rocprofv3's FETCH_SIZE / "
@@ -177,7 +180,8 @@ def bench_training(args):
             else:
                 g = (pred - yc) * lr
                 h = torch.ones_like(pred)
-            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed)
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed,
+                               hist_cache_bytes=args.hist_cache_bytes)
             pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
         else:
             # gradient step in one pass, which also leaves the first level of the quantiser's absolute
@@ -186,7 +190,7 @@ def bench_training(args):
             g, h, part = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc,
                                                pred, None, lr, out=gh, sums=sums)
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True, wait=False,
-                               abs_sum_chunks=part)
+                               abs_sum_chunks=part, hist_cache_bytes=args.hist_cache_bytes)
             ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         return r
 
@@ -278,6 +282,7 @@ def bench_training(args):
                         % (name, "LBClassifier softmax" if n_classes else "LBRegressor squared error", depth, S, lr,
                            n, f, k),
             "rows": n, "features": f, "outputs": k, "max_depth": depth, "split_samples": S,
+            "hist_cache_bytes": args.hist_cache_bytes or 1000000000,
             "loss_before": loss0, "loss_after": loss1,
             "prediction_update": "PredictTask" if args.reference_flow else "row->leaf map from BuildTreeTask",
             # a round as the reference loop runs it (legateboost.py:254-275): gradient arithmetic as

@@ -538,6 +538,10 @@ __global__ void __launch_bounds__(kThreads)
   if (threadIdx.x == 0) partial[static_cast<int64_t>(blockIdx.x) * n_chunks + blockIdx.y] = best;
 }
 
+// store == false: nothing reads these histograms after the split of their nodes has been applied
+// (the last level, or the level before one that starts a new histogram buffer), so the running
+// sums and the derived siblings are not written back; split_apply_kernel then forms the one bin
+// it needs from the bins as they were accumulated (stored_bin_value).
 // Scan, sibling subtraction and split evaluation in one pass over the histograms
 // (build_tree.cu:597-668 and :682-740): one wave per (built node, feature) takes 64 bins of the
 // feature at a time and, output by output, forms the running sums, stores them under the
@@ -581,7 +585,7 @@ __device__ inline Cand wave_best(Cand c)
 __global__ void __launch_bounds__(kThreads)
   scan_split_kernel(HistView hist, const I64Pair* node_sums, int F, const int32_t* row_pointers, int node_begin,
                     int n_nodes, const uint8_t* feature_set, const double* scales, double l1, double l2,
-                    double min_split_gain, Cand* partial)
+                    double min_split_gain, Cand* partial, bool store)
 {
   const int lane     = threadIdx.x & 63;
   const int64_t rank = (blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x) >> 6;
@@ -657,16 +661,16 @@ __global__ void __launch_bounds__(kThreads)
         // the reference skips the store when the running sum is not positive
         // (build_tree.cu:645); the raw bin value then stays in place
         if (in && (eg > 0 || eh > 0)) {
-          val                    = I64Pair{eg, eh};
-          *hist.at(node, k, bin) = val;
+          val = I64Pair{eg, eh};
+          if (store) *hist.at(node, k, bin) = val;
         }
         if (lane == k) {
           agg_g += tile_g;
           agg_h += tile_h;
         }
         if (derive && in) {
-          sval                  = I64Pair{sval.grad - val.grad, sval.hess - val.hess};
-          *hist.at(sib, k, bin) = sval;
+          sval = I64Pair{sval.grad - val.grad, sval.hess - val.hess};
+          if (store) *hist.at(sib, k, bin) = sval;
         }
       }
       if (eval_n && in) add_gain(gain_n, dead_n, val, ns, inv_g, inv_h, l1, reg, min_split_gain);
@@ -691,12 +695,35 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
+// What the reference's scan leaves in bin `bin` of (node, output k) of a built node whose bins still
+// hold what the rows added: the running sum over the feature's bins up to `bin` where that is
+// positive in either half, else the bin as it is (build_tree.cu:645); the bin as it is also where
+// the scan returns early for the output (:613). All 64 lanes call this together.
+__device__ inline I64Pair stored_bin_value(const HistView& hist, const I64Pair* node_sums, int node, int k, int fb,
+                                           int bin, int lane)
+{
+  const I64Pair raw = *hist.at(node, k, bin);
+  if (node_sums[static_cast<int64_t>(node) * hist.K + k].hess <= 0) return raw;
+  int64_t g = 0, h = 0;
+  for (int b = fb + lane; b <= bin; b += 64) {
+    const I64Pair p = *hist.at(node, k, b);
+    g += p.grad;
+    h += p.hess;
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    g += __shfl_xor(g, off, 64);
+    h += __shfl_xor(h, off, 64);
+  }
+  return (g > 0 || h > 0) ? I64Pair{g, h} : raw;
+}
+
+// stored == false: scan_split_kernel did not write its results back (see there).
 __global__ void __launch_bounds__(64)
   split_apply_kernel(HistView hist, I64Pair* node_sums, const int32_t* bin_feature,
                      const double* proposals_as_double, const double* scales, double l1, double l2,
                      int node_begin, int n_chunks, const Cand* partial, double* leaf,
                      int32_t* feature, double* split, double* gain_out, const int32_t* row_pointers,
-                     int32_t* split_bin)
+                     int32_t* split_bin, bool stored)
 {
   __shared__ Cand s_c[1];
   __shared__ Cand s_best;
@@ -715,6 +742,47 @@ __global__ void __launch_bounds__(64)
   if (!(best.bin >= 0 && best.gain > 1e-5)) return;
   const double inv_g = scales[2], inv_h = scales[3];
   const int lc = left_child(node), rc = right_child(node);
+  if (!stored) {
+    const int lane   = threadIdx.x;
+    const int ft     = bin_feature[best.bin];
+    const int fb     = row_pointers[ft];
+    const int parent = parent_of(node);
+    const bool built = compute_histogram_bin(node, node_sums, K, hist.contains(parent));
+    for (int k = 0; k < K; k++) {
+      const I64Pair ns = node_sums[static_cast<int64_t>(node) * K + k];
+      I64Pair ls;
+      if (built) {
+        ls = stored_bin_value(hist, node_sums, node, k, fb, best.bin, lane);
+      } else {
+        // derived from its parent and its built sibling, unless the scan of that sibling's output
+        // returned early: then the bin is what the buffer holds
+        const int sib = sibling_of(node);
+        if (node_sums[static_cast<int64_t>(sib) * K + k].hess > 0) {
+          const I64Pair sv = stored_bin_value(hist, node_sums, sib, k, fb, best.bin, lane);
+          const I64Pair pv = *hist.at(parent, k, best.bin);
+          ls               = I64Pair{pv.grad - sv.grad, pv.hess - sv.hess};
+        } else {
+          ls = *hist.at(node, k, best.bin);
+        }
+      }
+      if (lane == 0) {
+        const I64Pair rs{ns.grad - ls.grad, ns.hess - ls.hess};
+        node_sums[static_cast<int64_t>(lc) * K + k] = ls;
+        node_sums[static_cast<int64_t>(rc) * K + k] = rs;
+        leaf[static_cast<int64_t>(lc) * K + k]      = calculate_leaf_value(
+          static_cast<double>(ls.grad) * inv_g, static_cast<double>(ls.hess) * inv_h, l1, l2);
+        leaf[static_cast<int64_t>(rc) * K + k] = calculate_leaf_value(
+          static_cast<double>(rs.grad) * inv_g, static_cast<double>(rs.hess) * inv_h, l1, l2);
+        if (k == 0) {
+          feature[node]   = ft;
+          split[node]     = proposals_as_double[best.bin];
+          gain_out[node]  = best.gain;
+          split_bin[node] = best.bin - fb;
+        }
+      }
+    }
+    return;
+  }
   for (int k = threadIdx.x; k < K; k += 64) {
     I64Pair ns = node_sums[static_cast<int64_t>(node) * K + k];
     I64Pair ls = *hist.at(node, k, best.bin);
@@ -1707,12 +1775,19 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       // most of whose nodes are empty or small) the two kernels are faster: the evaluation then
       // runs over all bins of a node side by side, not feature by feature behind the scan.
       const bool fused = K <= kFusedMaxK && (K >= 2 || n_nodes <= 256);
+      // The scanned histograms of this level are read again only by the next level's sibling
+      // subtraction (and by a caller that asked to see them): not after the last level, and not
+      // when the next level starts a buffer of its own (GetHistogram, build_tree.cu:1191-1205).
+      const int64_t next_begin = level_begin(depth + 1), next_end = level_end(depth + 1);
+      const bool next_reads    = depth + 1 < max_depth && next_end - next_begin <= max_batch_size &&
+                              next_begin >= hv.node_begin && next_end <= hv.node_end;
+      const bool store = !fused || next_reads || (taps && taps->histogram);
       if (fused) {
         ProfScope ps(LBT_PROF_SCAN, stream);
         const int64_t waves = static_cast<int64_t>(F) * n_nodes;
         scan_split_kernel<<<blocks(waves, kThreads / 64), kThreads, 0, stream>>>(
           hv, L.node_sums, F, L.row_pointers, batch_begin, n_nodes, feature_set, L.scales, prm.l1_regularization,
-          prm.l2_regularization, prm.min_split_gain, L.partial);
+          prm.l2_regularization, prm.min_split_gain, L.partial, store);
       } else {
         {
           ProfScope ps(LBT_PROF_SCAN, stream);
@@ -1732,7 +1807,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
         split_apply_kernel<<<n_nodes, 64, 0, stream>>>(hv, L.node_sums, L.bin_feature, L.proposals_d, L.scales,
                                                        prm.l1_regularization, prm.l2_regularization, batch_begin,
                                                        n_cands, L.partial, leaf, feature, split, gain, L.row_pointers,
-                                                       L.split_bin);
+                                                       L.split_bin, store);
       }
     }
     if (depth < max_depth - 1) {

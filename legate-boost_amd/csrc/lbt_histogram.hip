@@ -61,51 +61,58 @@ __global__ void __launch_bounds__(kPlanThreads)
                     int K, int hist_node_begin, int hist_node_end, int tile_rows, int32_t* tile_start,
                     LevelMeta* meta, LevelMeta* level_total)
 {
+  // every thread owns a run of consecutive nodes: it counts their tiles, the workgroup scans the
+  // 256 counts once, and the thread walks its run again to write the starts
   __shared__ int s_scan[kPlanThreads];
-  __shared__ int s_run;
   __shared__ unsigned long long s_rb, s_rc, s_nb;
-  if (threadIdx.x == 0) {
-    s_run = 0;
-    s_rb = s_rc = s_nb = 0;
+  if (threadIdx.x == 0) s_rb = s_rc = s_nb = 0;
+  const int n     = j1 - j0;
+  const int per   = (n + kPlanThreads - 1) / kPlanThreads;
+  const int begin = j0 + min(n, static_cast<int>(threadIdx.x) * per);
+  const int end   = j0 + min(n, (static_cast<int>(threadIdx.x) + 1) * per);
+  auto tiles_of = [&](int j, int& rows, bool& built) {
+    const int node   = level_first + j;
+    rows             = seg[j + 1] - seg[j];
+    const int parent = parent_of(node);
+    const bool pex   = parent >= hist_node_begin && parent < hist_node_end;
+    built            = compute_histogram_bin(node, node_sums, K, pex);
+    return built ? (rows + tile_rows - 1) / tile_rows : 0;
+  };
+  int mine = 0;
+  unsigned long long rb = 0, rc = 0, nb = 0;
+  for (int j = begin; j < end; j++) {
+    int rows;
+    bool built;
+    mine += tiles_of(j, rows, built);
+    rb += static_cast<unsigned long long>(rows);
+    if (built && rows > 0) {
+      rc += static_cast<unsigned long long>(rows);
+      nb += 1;
+    }
   }
+  s_scan[threadIdx.x] = mine;
   __syncthreads();
-  for (int base = j0; base < j1; base += kPlanThreads) {
-    int j      = base + threadIdx.x;
-    int tiles  = 0;
-    int rows   = 0;
-    bool built = false;
-    if (j < j1) {
-      int node   = level_first + j;
-      rows       = seg[j + 1] - seg[j];
-      int parent = parent_of(node);
-      bool pex   = parent >= hist_node_begin && parent < hist_node_end;
-      built      = compute_histogram_bin(node, node_sums, K, pex);
-      tiles      = built ? (rows + tile_rows - 1) / tile_rows : 0;
-    }
-    s_scan[threadIdx.x] = tiles;
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    const int v = static_cast<int>(threadIdx.x) >= off ? s_scan[threadIdx.x - off] : 0;
     __syncthreads();
-    for (int off = 1; off < kPlanThreads; off <<= 1) {
-      int v = static_cast<int>(threadIdx.x) >= off ? s_scan[threadIdx.x - off] : 0;
-      __syncthreads();
-      s_scan[threadIdx.x] += v;
-      __syncthreads();
-    }
-    int run = s_run;
-    if (j < j1) {
-      tile_start[j - j0] = run + s_scan[threadIdx.x] - tiles;
-      atomicAdd(&s_rb, static_cast<unsigned long long>(rows));
-      if (built && rows > 0) {
-        atomicAdd(&s_rc, static_cast<unsigned long long>(rows));
-        atomicAdd(&s_nb, 1ULL);
-      }
-    }
-    __syncthreads();
-    if (threadIdx.x == kPlanThreads - 1) s_run = run + s_scan[kPlanThreads - 1];
+    s_scan[threadIdx.x] += v;
     __syncthreads();
   }
+  int run = s_scan[threadIdx.x] - mine;
+  for (int j = begin; j < end; j++) {
+    int rows;
+    bool built;
+    tile_start[j - j0] = run;
+    run += tiles_of(j, rows, built);
+  }
+  if (rb != 0) atomicAdd(&s_rb, rb);
+  if (rc != 0) atomicAdd(&s_rc, rc);
+  if (nb != 0) atomicAdd(&s_nb, nb);
+  __syncthreads();
   if (threadIdx.x == 0) {
-    tile_start[j1 - j0]   = s_run;
-    meta->n_tiles         = s_run;
+    const int total       = s_scan[kPlanThreads - 1];
+    tile_start[j1 - j0]   = total;
+    meta->n_tiles         = total;
     meta->instances       = s_rb;
     meta->built_instances = s_rc;
     meta->built_nodes     = s_nb;

@@ -136,6 +136,36 @@ def test_small_histogram_budget_batches():
         assert np.array_equal(gu.cpu(gr.feature), ref)
 
 
+@pytest.mark.parametrize("k,depth,budget", [(1, 5, 0), (3, 4, 0), (2, 5, 6000), (1, 6, 40000), (4, 1, 0), (2, 3, 1)])
+def test_tree_without_histogram_tap_matches_oracle(k, depth, budget):
+    """A caller that does not ask for the histograms lets the last level (and a level before a new
+    histogram buffer) keep its running sums to itself: the tree must be the one the oracle builds, with
+    l1 regularisation, a minimum gain, outputs whose hessian sums vanish in some nodes and empty nodes."""
+    import gpu_util as gu
+    import oracle_lib as orc
+    from lbtree import ops
+
+    X, g, h = _problem(40 + k, 4000, 9, k)
+    # a few rows carry all the hessian mass of the last output: its sums vanish in most nodes
+    if k > 1:
+        h[:, k - 1] = 0.0
+        h[:40, k - 1] = 1.0
+    kw = dict(max_depth=depth, split_samples=32, seed=77, l1_regularization=0.01, min_split_gain=1e-4,
+              hist_cache_bytes=budget)
+    cr = orc.build_tree(X, g, h, max_depth=depth, split_samples=32, seed=77, l1=0.01, l2=1.0, min_split_gain=1e-4,
+                        hist_cache_bytes=budget)
+    plain = ops.build_tree(X, g, h, row_leaf=True, **kw)
+    tapped = ops.build_tree(X, g, h, taps=True, row_leaf=True, **kw)
+    gu.assert_tree_parity(tapped, cr)
+    for got in (plain, tapped):
+        assert np.array_equal(gu.cpu(got.feature), cr.feature)
+        gu.assert_same_floats(gu.cpu(got.split_value), cr.split_value, "split_value")
+        gu.assert_same_floats(gu.cpu(got.gain), cr.gain, "gain")
+        gu.assert_same_floats(gu.cpu(got.leaf_value), cr.leaf_value, "leaf_value")
+        gu.assert_same_floats(gu.cpu(got.hessian), cr.hessian, "hessian")
+    assert np.array_equal(gu.cpu(plain.row_leaf), gu.cpu(tapped.row_leaf))
+
+
 def test_deep_tree_with_duplicates_and_small_nodes():
     import gpu_util as gu
 
