@@ -167,7 +167,7 @@ def bench_training(args):
     gh = (torch.empty_like(pred), torch.empty_like(pred))
     sums = torch.empty((2, int(_lib.lib.lbt_abs_sum_chunks(n, k))), dtype=torch.float64, device=X.device)
 
-    def one_round(reference_flow=args.reference_flow):
+    def one_round(reference_flow=args.reference_flow, cache=args.hist_cache_bytes):
         seed = int(rs.randint(0, 2**31))
         if reference_flow:
             # the caller's steps as separate array operations and a traversal of X per round
@@ -180,8 +180,7 @@ def bench_training(args):
             else:
                 g = (pred - yc) * lr
                 h = torch.ones_like(pred)
-            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed,
-                               hist_cache_bytes=args.hist_cache_bytes)
+            r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, hist_cache_bytes=cache)
             pred.add_(ops.predict(X, [(r.leaf_value, r.feature, r.split_value)], k))
         else:
             # gradient step in one pass, which also leaves the first level of the quantiser's absolute
@@ -190,7 +189,7 @@ def bench_training(args):
             g, h, part = ops.weighted_gradient("log_loss" if n_classes else "squared_error", y if n_classes else yc,
                                                pred, None, lr, out=gh, sums=sums)
             r = ops.build_tree(X, g, h, max_depth=depth, split_samples=S, seed=seed, row_leaf=True, wait=False,
-                               abs_sum_chunks=part, hist_cache_bytes=args.hist_cache_bytes)
+                               abs_sum_chunks=part, hist_cache_bytes=cache)
             ops.add_leaf_values(pred, r.leaf_value, r.row_leaf)
         return r
 
@@ -232,6 +231,20 @@ def bench_training(args):
         one_round(not args.reference_flow)
     torch.cuda.synchronize()
     other_rate = other_steps / (time.perf_counter() - t0)
+
+    # The reference keeps 1e9 bytes of histograms (build_tree.cu:1004); a tree whose levels outgrow that
+    # builds both children of every node from there on. With room for the whole tree (this GPU has 288 GB)
+    # the same trees come out and every level derives siblings by subtraction: measured in the same run.
+    whole_tree = (2 ** depth - 1) * k * f * S * 16
+    whole_rate = None
+    if whole_tree > (args.hist_cache_bytes or 1000000000):
+        one_round(cache=whole_tree)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(other_steps):
+            one_round(cache=whole_tree)
+        torch.cuda.synchronize()
+        whole_rate = other_steps / (time.perf_counter() - t0)
 
     hist, binning = prof["histogram"], prof["binning"]
     elem = X.element_size()
@@ -290,6 +303,8 @@ def bench_training(args):
             "reference_flow_rounds_per_s": args.steps / dt if args.reference_flow else other_rate,
             "fused_flow_rounds_per_s": other_rate if args.reference_flow else args.steps / dt,
             "other_flow_steps": other_steps,
+            "rounds_per_s_with_histograms_of_the_whole_tree_cached": whole_rate,
+            "whole_tree_histogram_bytes": whole_tree,
         },
         # the kernel with the largest share of a round: the histogram kernel on cached bins,
         # priced on the bytes of its own input format (one or two bytes per feature value)
@@ -373,10 +388,19 @@ def bench_predict(args):
         "config": {"workload": "cfg5: PredictTask, 1000 trees of depth 8, X %dx64 f32, out f64" % rows,
                    "rows": rows, "trees": 1000, "row_trees_per_s": rows * 1000 * args.steps / dt,
                    "node_steps_per_s": rows * 8000 * args.steps / dt},
-        # X read once and the output written once are all the HBM bytes this path needs; the
-        # kernel's own limit is the 8000 node steps per row, served from LDS
+        # X read once and the output written once are all the HBM bytes this path needs (achieved /
+        # peak / frac price those); what bounds the kernel is the LDS: every node step of a wave
+        # is two LDS reads (node, feature value), which the counters put at 8.2 cycles each
+        # (4.2 of issue, 3.4 of bank conflicts; profiles/predict_tile_kernel_cfg5_*.txt), 17 of
+        # the 17.5 cycles a CU spends per wave-level node step
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "predict_tile_kernel"},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": "predict_tile_kernel",
+                     "limited_by": "lds",
+                     "lds": {"wave_level_node_steps": rows * 8000 / 64,
+                             "cycles_per_wave_level_node_step_and_cu":
+                                 dt / args.steps * 2.4e9 / (rows * 8000 / 64 / 256),
+                             "lds_reads_per_node_step": 2.1, "lds_cycles_per_read_measured": 8.2,
+                             "clock_assumed_GHz": 2.4}},
     }
     if not args.no_cpu_baseline:
         cores = max(1, min(16, os.cpu_count() or 1))
