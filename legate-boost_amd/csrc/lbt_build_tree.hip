@@ -64,8 +64,11 @@ __device__ inline void atomic_add_i64(int64_t* p, int64_t v)
 // tree initialisation / output (build_tree.cu:785-861)
 // ---------------------------------------------------------------------------
 
+// Also what the TreeBuilder's constructor sets up (build_tree.cu:967-974, every row starts in the
+// root) and the per-level counters, so that a tree starts with one launch instead of three.
 __global__ void init_tree_kernel(double* leaf, int32_t* feature, double* split, double* gain,
-                                 I64Pair* node_sums, int64_t max_nodes, int K)
+                                 I64Pair* node_sums, int64_t max_nodes, int K, int32_t* rows, int64_t n, int32_t* seg,
+                                 int32_t* block_seg, int64_t n_slabs, uint4* level_totals, int n_totals16)
 {
   int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
   if (i < max_nodes * K) {
@@ -76,6 +79,13 @@ __global__ void init_tree_kernel(double* leaf, int32_t* feature, double* split, 
     feature[i] = -1;
     split[i]   = 0.0;
     gain[i]    = 0.0;
+  }
+  if (i < n) rows[i] = static_cast<int32_t>(i);
+  if (i < n_slabs) block_seg[i] = 0;
+  if (i < n_totals16) level_totals[i] = make_uint4(0, 0, 0, 0);
+  if (i == 0) {
+    seg[0] = 0;
+    seg[1] = static_cast<int32_t>(n);
   }
 }
 
@@ -176,22 +186,37 @@ __global__ void __launch_bounds__(kThreads)
 }
 
 // CSR row pointers (reduce_by_key + inclusive_scan, build_tree.cu:933-949)
-__global__ void row_pointers_kernel(const int32_t* counts, int F, int32_t* row_pointers)
+// One workgroup: every thread adds up a run of consecutive counts, the runs are joined by a scan
+// over the workgroup, and the thread walks its run again to write the pointers.
+__global__ void __launch_bounds__(kThreads) row_pointers_kernel(const int32_t* counts, int F, int32_t* row_pointers)
 {
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    int run         = 0;
-    row_pointers[0] = 0;
-    for (int f = 0; f < F; f++) {
-      run += counts[f];
-      row_pointers[f + 1] = run;
-    }
+  __shared__ int s_scan[kThreads];
+  const int per   = (F + kThreads - 1) / kThreads;
+  const int begin = min(F, static_cast<int>(threadIdx.x) * per);
+  const int end   = min(F, begin + per);
+  int mine = 0;
+  for (int f = begin; f < end; f++) mine += counts[f];
+  s_scan[threadIdx.x] = mine;
+  __syncthreads();
+  for (int off = 1; off < kThreads; off <<= 1) {
+    const int v = static_cast<int>(threadIdx.x) >= off ? s_scan[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_scan[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int run = s_scan[threadIdx.x] - mine;
+  if (threadIdx.x == 0) row_pointers[0] = 0;
+  for (int f = begin; f < end; f++) {
+    run += counts[f];
+    row_pointers[f + 1] = run;
   }
 }
 
 // compact copy; the last proposal of each feature becomes +inf (build_tree.cu:953-956)
+// as_double (optional): the same values as doubles, what WriteTreeOutput stores as split values
 template <typename T>
 __global__ void compact_proposals_kernel(const T* uniq, int S, const int32_t* row_pointers,
-                                         T* proposals, int32_t* bin_feature)
+                                         T* proposals, int32_t* bin_feature, double* as_double)
 {
   const int f = blockIdx.x;
   int b0 = row_pointers[f], b1 = row_pointers[f + 1];
@@ -200,6 +225,7 @@ __global__ void compact_proposals_kernel(const T* uniq, int S, const int32_t* ro
     if (i == b1 - b0 - 1) v = std::numeric_limits<T>::infinity();
     proposals[b0 + i]   = v;
     bin_feature[b0 + i] = f;
+    if (as_double != nullptr) as_double[b0 + i] = static_cast<double>(v);
   }
 }
 
@@ -803,12 +829,6 @@ __global__ void __launch_bounds__(64)
   }
 }
 
-template <typename T>
-__global__ void proposals_to_double_kernel(const T* p, int n, double* out)
-{
-  int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) out[i] = static_cast<double>(p[i]);
-}
 
 // ---------------------------------------------------------------------------
 // row -> node update and stable partition (build_tree.cu:1026-1080)
@@ -1345,18 +1365,6 @@ __global__ void __launch_bounds__(kThreads)
   }
 }
 
-// build_tree.cu:967-974: every row starts in the root
-__global__ void fill_positions_kernel(int32_t* rows, int64_t n, int32_t* seg, int32_t* block_seg, int64_t n_slabs)
-{
-  int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
-  if (i < n) rows[i] = static_cast<int32_t>(i);
-  if (i < n_slabs) block_seg[i] = 0;
-  if (i == 0) {
-    seg[0] = 0;
-    seg[1] = static_cast<int32_t>(n);
-  }
-}
-
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -1550,7 +1558,7 @@ int host_mirror(int F, ThreadResources** out)
 template <typename T>
 int run_split_samples(hipStream_t stream, const T* X, int64_t row_offset, int64_t N, int F, int S, int32_t seed,
                       int64_t dataset_rows, T* draft, T* uniq, int32_t* counts, int32_t* row_pointers, T* proposals,
-                      int32_t* bin_feature)
+                      int32_t* bin_feature, double* proposals_as_double = nullptr)
 {
   auto blocks = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
   gather_samples_kernel<T><<<blocks(static_cast<int64_t>(F) * S, kThreads), kThreads, 0, stream>>>(
@@ -1559,8 +1567,9 @@ int run_split_samples(hipStream_t stream, const T* X, int64_t row_offset, int64_
   while (P < S) P <<= 1;
   if (P < 2) P = 2;
   sort_unique_kernel<T><<<F, kThreads, P * sizeof(typename KeyOf<T>::type), stream>>>(draft, S, P, uniq, counts);
-  row_pointers_kernel<<<1, 64, 0, stream>>>(counts, F, row_pointers);
-  compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(uniq, S, row_pointers, proposals, bin_feature);
+  row_pointers_kernel<<<1, kThreads, 0, stream>>>(counts, F, row_pointers);
+  compact_proposals_kernel<T><<<F, kThreads, 0, stream>>>(uniq, S, row_pointers, proposals, bin_feature,
+                                                          proposals_as_double);
   LBT_HIP(hipGetLastError());
   return LBT_OK;
 }
@@ -1623,8 +1632,12 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
 
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
-    init_tree_kernel<<<blocks(static_cast<int64_t>(max_nodes) * K, kThreads), kThreads, 0, stream>>>(
-      leaf, feature, split, gain, L.node_sums, max_nodes, K);
+    static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
+    const int64_t n_slabs = (N + kPartBlock - 1) / kPartBlock;
+    const int64_t widest  = std::max<int64_t>(std::max<int64_t>(static_cast<int64_t>(max_nodes) * K, N), 2 * max_depth);
+    init_tree_kernel<<<blocks(std::max<int64_t>(widest, 1), kThreads), kThreads, 0, stream>>>(
+      leaf, feature, split, gain, L.node_sums, max_nodes, K, L.rows[0], N, L.seg[0], L.block_seg[0], n_slabs,
+      reinterpret_cast<uint4*>(L.level_totals), std::max(0, max_depth * 2));
   }
 
   // ---- split proposals
@@ -1635,7 +1648,7 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
     ProfScope ps(LBT_PROF_PROPOSALS, stream);
     LBT_TRY(run_split_samples<T>(stream, X, row_offset, N, F, S, prm.seed, prm.dataset_rows, static_cast<T*>(L.draft),
                                  static_cast<T*>(L.uniq), L.counts, L.row_pointers, static_cast<T*>(L.proposals),
-                                 L.bin_feature));
+                                 L.bin_feature, L.proposals_d));
     LBT_HIP(hipMemcpyAsync(rp_here, L.row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, stream));
     LBT_HIP(hipEventRecord(hm->counts_here, stream));
   }
@@ -1666,10 +1679,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   };
 
   // ---- positions and histogram cache (TreeBuilder ctor, build_tree.cu:997-1017)
-  fill_positions_kernel<<<blocks(N, kThreads), kThreads, 0, stream>>>(L.rows[0], N, L.seg[0], L.block_seg[0],
-                                                                       (N + kPartBlock - 1) / kPartBlock);
-  static_assert(sizeof(LevelMeta) == 32, "LevelMeta is cleared in 16-byte units");
-  if (max_depth > 0) zero_kernel<<<1, kThreads, 0, stream>>>(reinterpret_cast<uint4*>(L.level_totals), max_depth * 2);
 
   // the one host wait before the levels: the bin counts decide the feature groups. Only the
   // copy of the counts is waited for; the quantiser queued behind it keeps the GPU busy while
@@ -1677,8 +1686,6 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
   LBT_HIP(hipEventSynchronize(hm->counts_here));
   const std::vector<int32_t> rp(rp_here, rp_here + F + 1);
   const int B = rp[F];
-  proposals_to_double_kernel<T><<<blocks(B, kThreads), kThreads, 0, stream>>>(
-    static_cast<const T*>(L.proposals), B, L.proposals_d);
 
   HistSetup hs;
   hs.groups     = L.groups;
