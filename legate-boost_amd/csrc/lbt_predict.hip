@@ -223,29 +223,32 @@ __global__ void write_batches_kernel(BatchTable t, int first, int n, BatchInfo* 
   if (i < n) out[first + i] = t.b[i];
 }
 
-// Every lane of a group of L lanes reads lane kLane of its group (groups of four through a
-// quad permute, wider ones through a lane-indexed shuffle).
-template <int L, int kLane>
-__device__ inline int group_broadcast(int v)
+// The L lanes of a row sit 64 / L lanes apart in their wave: lane = q * (64 / L) + (row of the wave),
+// q the row's lane. A quarter wave (what the LDS serves at once) then holds lanes that walk the same
+// tree for neighbouring rows: they read neighbouring nodes and, while they agree on the feature,
+// neighbouring feature values, where the lanes of one row side by side would read four unrelated trees.
+// Lane q of a row owns the trees q * kLaneTrees .. of a batch.
+template <int L>
+__device__ inline int from_previous_lane_of_row(int v)
 {
-  if constexpr (L == 4)
-    return __builtin_amdgcn_mov_dpp(v, kLane * 0x55, 0xf, 0xf, false);
-  else
-    return __shfl(v, (static_cast<int>(threadIdx.x) & 63 & ~(L - 1)) | kLane, 64);
+  // value of the lane 64 / L below (the row's lane q - 1; lane 0 of a row reads its last lane)
+  return __shfl(v, (static_cast<int>(threadIdx.x) + 64 - 64 / L) & 63, 64);
 }
-template <int L, int kLane>
-__device__ inline double group_broadcast(double v)
+template <int L>
+__device__ inline double from_previous_lane_of_row(double v)
 {
   const long long bits = __double_as_longlong(v);
-  const int lo = group_broadcast<L, kLane>(static_cast<int>(bits));
-  const int hi = group_broadcast<L, kLane>(static_cast<int>(bits >> 32));
+  const int lo = from_previous_lane_of_row<L>(static_cast<int>(bits));
+  const int hi = from_previous_lane_of_row<L>(static_cast<int>(bits >> 32));
   return __longlong_as_double((static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
 }
-// value of tree jj of a batch, held by lane jj % L of the row's lanes in slot jj / L
-template <typename S, int jj, typename V>
-__device__ inline V from_owner(const V (&slots)[S::kLaneTrees])
+// value of tree jj of a batch, held by lane jj / kLaneTrees of the row's lanes in slot jj % kLaneTrees
+template <typename S, int jj>
+__device__ inline int from_owner(const int (&slots)[S::kLaneTrees])
 {
-  return group_broadcast<S::kRowLanes, jj % S::kRowLanes>(slots[jj / S::kRowLanes]);
+  constexpr int kStride = 64 / S::kRowLanes;
+  const int row_in_wave = static_cast<int>(threadIdx.x) & (kStride - 1);
+  return __shfl(slots[jj % S::kLaneTrees], (jj / S::kLaneTrees) * kStride + row_in_wave, 64);
 }
 
 // What is fetched one batch ahead: the nodes as 16-byte words and where this lane's trees start
@@ -275,37 +278,30 @@ __device__ __forceinline__ Prefetched<S> fetch_batch(const BatchInfo& bi, const 
   }
 #pragma unroll
   for (int j = 0; j < S::kLaneTrees; j++) {
-    const int jj = q + S::kRowLanes * j;
+    const int jj = q * S::kLaneTrees + j;
     pf.base[j]   = desc[bi.first + (jj < bi.count ? jj : 0)].rel_off;  // lanes without a tree walk tree 0 again
   }
   return pf;
 }
 
-template <typename S, int jj>
-__device__ __forceinline__ void add_in_order_from(double& acc, const double (&val)[S::kLaneTrees], int cnt)
-{
-  if constexpr (jj < S::kBatchTrees) {
-    const double v = from_owner<S, jj>(val);
-    if (jj < cnt) acc += v;
-    add_in_order_from<S, jj + 1>(acc, val, cnt);
-  }
-}
-template <typename S, int jj>
-__device__ __forceinline__ void add_all_in_order_from(double& acc, const double (&val)[S::kLaneTrees])
-{
-  if constexpr (jj < S::kBatchTrees) {
-    acc += from_owner<S, jj>(val);
-    add_all_in_order_from<S, jj + 1>(acc, val);
-  }
-}
+// Single output: the sum of a row travels along the row's lanes. Lane 0 takes what the last lane
+// holds (the sum up to the previous batch), adds the leaf values of its own trees in tree order and
+// hands the sum on; after the last lane's turn that lane holds the sum up to this batch. Every lane
+// runs every turn (the lanes whose turn it is not keep their value), so the adds of a row happen in
+// tree order exactly as the per-tree launches of the reference add them.
 template <typename S>
-__device__ __forceinline__ void add_in_order(double& acc, const double (&val)[S::kLaneTrees], int cnt)
+__device__ __forceinline__ void add_in_order(double& run, const double (&val)[S::kLaneTrees], int cnt, int q)
 {
-  // all batches but the last are full: no test per tree then
-  if (cnt == S::kBatchTrees)
-    add_all_in_order_from<S, 0>(acc, val);
-  else
-    add_in_order_from<S, 0>(acc, val, cnt);
+#pragma unroll
+  for (int turn = 0; turn < S::kRowLanes; turn++) {
+    double t = from_previous_lane_of_row<S::kRowLanes>(run);
+#pragma unroll
+    for (int j = 0; j < S::kLaneTrees; j++) {
+      const double a = t + val[j];
+      t              = q * S::kLaneTrees + j < cnt ? a : t;
+    }
+    run = q == turn ? t : run;
+  }
 }
 template <typename S, int kAcc, int jj>
 __device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
@@ -369,8 +365,9 @@ __global__ void __launch_bounds__(kTileThreads)
       }
     }
   }
-  const int r      = threadIdx.x / L;
-  const int q      = threadIdx.x & (L - 1);
+  constexpr int kRowsPerWave = 64 / L;
+  const int r      = (static_cast<int>(threadIdx.x) >> 6) * kRowsPerWave + (static_cast<int>(threadIdx.x) & (kRowsPerWave - 1));
+  const int q      = (static_cast<int>(threadIdx.x) & 63) / kRowsPerWave;
   const bool valid = r < rows_here;
   const T* my_x    = s_x + (valid ? r : 0) * pitch;
   constexpr int kAcc = kSingle ? 1 : kTileMaxK;
@@ -424,9 +421,8 @@ __global__ void __launch_bounds__(kTileThreads)
       }
     }
     if constexpr (kSingle) {
-      // leaf values of the previous batch arrived while this one was walked: every lane of the
-      // four forms the same sum, in tree order
-      add_in_order<S>(acc[0], val, cnt_prev);
+      // leaf values of the previous batch arrived while this one was walked
+      add_in_order<S>(acc[0], val, cnt_prev, q);
 #pragma unroll
       for (int j = 0; j < kLaneTrees; j++) val[j] = leaves[info.node_off + base[j] + pos[j]];
       cnt_prev = info.count;
@@ -437,8 +433,9 @@ __global__ void __launch_bounds__(kTileThreads)
       add_leaves_in_order<S, kAcc>(acc, at, info.count, leaves + info.node_off * K, K);
     }
   }
-  if constexpr (kSingle) add_in_order<S>(acc[0], val, cnt_prev);
-  if (valid && q == 0) {
+  if constexpr (kSingle) add_in_order<S>(acc[0], val, cnt_prev, q);
+  // single output: the row's last lane holds the sum; several outputs: every lane of the row does
+  if (valid && q == (kSingle ? L - 1 : 0)) {
     double* o = out + (row0 + r) * K;
 #pragma unroll
     for (int k = 0; k < kAcc; k++)
