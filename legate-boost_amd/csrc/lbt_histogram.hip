@@ -420,8 +420,9 @@ struct Stripes {
 // Merge of a striped sub-histogram into the int64 histogram of a node; s_off[p] is the place of
 // feature p's first bin in the group's run of bins.
 // sole_owner: no other workgroup adds to these bins and nothing has been added to them yet (the
-// histogram starts from zero and the parked parts of a node are added after the launch): the
-// sums are stored as they are, which neither waits for a load nor occupies the L2's atomic units.
+// histogram starts from zero, parked parts of a node are added after the launch, and the caller
+// does not claim ownership of a node of which it has already merged a part): the sums are stored
+// as they are, which neither waits for a load nor occupies the L2's atomic units.
 __device__ inline void merge_striped(unsigned long long* s_hist, const Stripes& st, const int* s_off, I64Pair* dst,
                                      bool sole_owner, int gs)
 {
@@ -468,9 +469,8 @@ __device__ inline void park_sub_histogram(unsigned long long* s_hist, int nb, I6
     return;
   }
   if (sole_owner) {
-    // every row of the node went through this workgroup: nobody else adds to these bins, and
-    // nothing has been added to them yet (the histogram starts from zero, parked parts of the
-    // node are added after the launch), so the sums are stored as they are
+    // every row of the node went through this workgroup in one piece: nobody else adds to these
+    // bins, and nothing has been added to them yet, so the sums are stored as they are
     for (int i = threadIdx.x; i < nb; i += kHistThreads) {
       const unsigned long long v = s_hist[i];
       if (v != 0) {
@@ -1197,8 +1197,12 @@ __global__ void __launch_bounds__(kHistThreads)
   unsigned long long acc = 0;
   // rows of cur_node that this workgroup has taken, and how many the node has: when they
   // agree at the end of the node, its bins belong to this workgroup alone. Not when single
-  // tiles may go to the histogram directly (huge gradients), which other workgroups may do too.
+  // tiles may go to the histogram directly (huge gradients), which other workgroups may do too,
+  // and not when a part of the node has left the LDS before its end (node_flushed): without a
+  // free slot that part was added to the histogram with atomics during this launch, and a plain
+  // store of the rest would overwrite it.
   int node_rows = 0, node_total = 0;
+  bool node_flushed = false;
   const bool owners = static_cast<unsigned long long>(w.tile_rows) * max_abs <= 2147483647ULL;
   __syncthreads();
 
@@ -1283,8 +1287,10 @@ __global__ void __launch_bounds__(kHistThreads)
         if (cur_node >= 0)
           park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink,
                              (cur_node - w.level_first - w.j0) * w.n_gk + gk, &s_slot,
-                             owners && tc.node != cur_node && node_rows == node_total, st, s_off, gs);
+                             owners && tc.node != cur_node && !node_flushed && node_rows == node_total, st, s_off,
+                             gs);
         __syncthreads();
+        node_flushed = tc.node == cur_node;
         if (tc.node != cur_node) {
           node_rows  = 0;
           node_total = tc.seg_rows;
@@ -1413,7 +1419,7 @@ __global__ void __launch_bounds__(kHistThreads)
   __syncthreads();
   if (cur_node >= 0)
     park_sub_histogram(s_hist, nb, a.hist.at(cur_node, k, bin0), sink, (cur_node - w.level_first - w.j0) * w.n_gk + gk,
-                       &s_slot, owners && node_rows == node_total, st, s_off, gs);
+                       &s_slot, owners && !node_flushed && node_rows == node_total, st, s_off, gs);
 }
 
 template <typename T, int VEC, bool kIdentityRows>

@@ -63,6 +63,24 @@ def _subsample_parity(X, g, h, rows, **kw):
     return gr, cr
 
 
+def test_config2_first_rows_bit_exact():
+    """The headline shape: 100 features (two feature groups of 52 and 48 whose records carry the
+    gradient pair), one output, depth 8, 256 split samples, on the first 200,000 rows of the
+    10,000,000 x 100 matrix, level by level against the oracle."""
+    from lbtree import datasets
+
+    X, y = datasets.config2(10_000_000, 100)
+    assert X.shape == (10_000_000, 100)
+    g, h = _squared_error_gradients(y)
+    gr, cr = _subsample_parity(X, g, h, 200_000, max_depth=8, split_samples=256, seed=24680)
+    assert (cr.hist_node_begin, cr.hist_node_end) == (0, 1023)  # 2441 nodes of 25,600 bins fit the cache
+    assert np.diff(cr.row_pointers).max() == 256
+    assert (cr.feature != -1).sum() > 200
+    # siblings are derived by subtraction from level 1 on
+    for d in range(1, 8):
+        assert cr.level_built_instances[d] < (cr.positions_per_level[d][:, 0] >= 0).sum()
+
+
 def test_config3_first_rows_bit_exact(config3):
     """200 features, 8 softmax outputs, depth 8, 256 split samples; the oracle takes about 20 s."""
     X, g, h = config3

@@ -60,6 +60,65 @@ def test_every_scanned_feature_ends_in_the_node_sum(built):
     assert torch.equal(ends[reached], sums[reached].unsqueeze(1).expand(-1, len(rp) - 1, -1))
 
 
+def _best_split_on_the_host(hist, sums, rp, scales):
+    """perform_best_split (build_tree.cu:682-782) of one node from its scanned histogram
+    [bins][2] and its sums [2], one output, no feature set, l1 = 0, l2 = 1, min_split_gain = 0:
+    the gain of every bin with the oracle's scalar, zero where a child has no hessian, then the
+    arg-max under the reference's order (strictly greater gain wins inside each of its 512 strided
+    threads, so the lowest bin of a residue class; the rank-ordered reduce keeps the later class on
+    ties, so the highest residue). Returns (bin, gain) or (-1, 0.0)."""
+    import oracle_lib as orc
+
+    lib = orc._load()
+    ng, nh = int(sums[0]), int(sums[1])
+    gains = np.zeros(len(hist))
+    for b in range(len(hist)):
+        lg, lh = int(hist[b, 0]), int(hist[b, 1])
+        rg, rh = ng - lg, nh - lh
+        if lh <= 0 or rh <= 0:
+            continue
+        gains[b] = lib.orc_calculate_gain(lg * scales[2], lh * scales[3], rg * scales[2], rh * scales[3],
+                                          ng * scales[2], nh * scales[3], 0.0, 1.0, 0.0)
+    top = gains.max()
+    if not top > 1e-5:
+        return -1, 0.0
+    tied = np.flatnonzero(gains == top)
+    residue = (tied % 512).max()
+    return int(tied[tied % 512 == residue].min()), float(top)
+
+
+def test_split_decisions_follow_from_the_histograms(built):
+    """Root and two nodes of each deeper level: feature, threshold and gain recomputed on the
+    host from the node's scanned histogram (itself checked against a direct count above)."""
+    _, _, _, r = built
+    rp = r.row_pointers.cpu().numpy()
+    feature = r.feature.cpu().numpy()
+    split = r.split_value.cpu().numpy()
+    gain = r.gain.cpu().numpy()
+    sums = r.node_sums.cpu().numpy()
+    proposals = r.proposals.cpu().numpy()
+    assert r.hist_node_begin == 0
+    checked = 0
+    for d in range(8):
+        first = 2 ** d - 1
+        level = [n for n in range(first, 2 * first + 1) if sums[n, 0, 1] > 0]
+        for node in sorted({level[0], level[len(level) // 2], level[-1]}):
+            hist = r.histogram[node, 0].cpu().numpy()
+            b, top = _best_split_on_the_host(hist, sums[node, 0], rp, r.scales)
+            if b < 0:
+                assert feature[node] == -1
+                continue
+            f = int(np.searchsorted(rp, b, side="right") - 1)
+            assert feature[node] == f, (node, feature[node], f)
+            assert split[node] == float(proposals[b]), node
+            assert gain[node] == top, node
+            # the children's sums are the chosen bin and what is left of the node
+            assert np.array_equal(sums[2 * node + 1, 0], hist[b])
+            assert np.array_equal(sums[2 * node + 2, 0], sums[node, 0] - hist[b])
+            checked += 1
+    assert checked >= 15
+
+
 def test_positions_are_a_stable_partition(built):
     X, _, _, r = built
     pos = r.positions.to(torch.int64)
