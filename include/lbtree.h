@@ -209,6 +209,73 @@ int lbt_quantise_gradients_static(void* stream, const double* g, const double* h
                                   int32_t n_outputs, int64_t row_offset, int32_t seed, int32_t* quantised,
                                   int64_t* root_sums, double* scales);
 
+/*
+ * The four stages of one tree level on their own, at the places where the reference cuts its
+ * level (build_tree.cu:1082-1124 histogram | scan, :1126-1152 best split, :1026-1080 positions), on
+ * the reference's own layouts, so that each can be compared and timed alone:
+ *   histogram  device int64 [hist_node_end - hist_node_begin][n_outputs][n_bins][2] (grad, hess), the
+ *              Histogram of build_tree.h:231-306 for the nodes [hist_node_begin, hist_node_end)
+ *   positions  device int32 [n_rows][2] of (node, row), sorted by node, retired rows (node -1)
+ *              in front: sorted_positions of build_tree.cu:997-1001
+ *   node_sums  device int64 [nodes][n_outputs][2], nodes at least 2 * batch_end + 1 where children
+ *              are written
+ *   proposals, row_pointers  as lbt_select_split_samples leaves them; n_bins = row_pointers[n_features]
+ *   quantised, scales        as lbt_quantise_gradients leaves them
+ *   [batch_begin, batch_end) the nodes of the call: all of one level, or a part of it
+ * They run the kernels of lbt_build_tree (which fuses some of them and keeps the order as row
+ * numbers plus segment starts; here the (node, row) pairs are converted on the way in and out).
+ * All of them enqueue on the stream; lbt_histogram_level and lbt_update_positions wait once for a
+ * check of their input.
+ *
+ * HistogramKernel (build_tree.cu:213-577): every row of a node of the batch whose histogram is
+ * built (ComputeHistogramBin, build_tree.h:92-104: the root, every node whose parent is not in
+ * [hist_node_begin, hist_node_end), else the child with the smaller sum of hessians) adds its
+ * quantised pair to the bin of each of its feature values. Sums are added to `histogram`, which the
+ * caller has cleared (the reference clears it when it allocates it, build_tree.cu:1012, :1198).
+ *   split_samples  upper bound on the proposals of one feature (sizes the workspace)
+ *   level          tree level of the batch; every pair of `positions` is of that level or retired
+ *   reuse_bins     non-zero: the workspace still holds the cached bins that an earlier call with the
+ *                  same X, proposals, split_samples and workspace left there (the binning pass is
+ *                  skipped); zero: X is binned first
+ */
+size_t lbt_histogram_level_workspace_bytes(int64_t n_rows, int32_t n_features, int32_t split_samples, int32_t x_dtype,
+                                           int32_t level);
+int lbt_histogram_level(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                        const int32_t* quantised, int32_t n_outputs, const void* proposals,
+                        const int32_t* row_pointers, int32_t split_samples, const int32_t* positions, int32_t level,
+                        int32_t batch_begin, int32_t batch_end, const int64_t* node_sums, int32_t hist_node_begin,
+                        int32_t hist_node_end, int64_t* histogram, void* workspace, size_t workspace_bytes,
+                        int32_t reuse_bins);
+
+/* scan_kernel (build_tree.cu:597-668): in place, per built node, output and feature the running
+ * sums over the feature's bins (a bin is left as it is where neither running sum is positive,
+ * :645; outputs whose node sum of hessians is not positive are skipped, :613), then the bins of a
+ * sibling that is not built as parent minus node. */
+int lbt_scan(void* stream, int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end, int32_t n_outputs,
+             int32_t n_features, const int32_t* row_pointers, int32_t n_bins, const int64_t* node_sums,
+             int32_t batch_begin, int32_t batch_end);
+
+/* perform_best_split (build_tree.cu:682-782) on a scanned histogram: for every node of the batch
+ * with a positive sum of hessians the bin of the largest gain under the reference's order among
+ * equal gains; where that gain exceeds 1e-5 it writes feature, split and gain of the node and
+ * node_sums and leaf of its two children. leaf is [nodes][n_outputs]; feature, split, gain [nodes]. */
+size_t lbt_best_split_workspace_bytes(int32_t n_features, int32_t n_bins, int32_t batch_begin, int32_t batch_end);
+int lbt_best_split(void* stream, const int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end,
+                   int32_t n_outputs, int32_t n_features, const void* proposals, int32_t x_dtype,
+                   const int32_t* row_pointers, int32_t n_bins, const uint8_t* feature_set, int64_t* node_sums,
+                   const double* scales, double l1_regularization, double l2_regularization, double min_split_gain,
+                   int32_t batch_begin, int32_t batch_end, double* leaf, int32_t* feature, double* split, double* gain,
+                   void* workspace, size_t workspace_bytes);
+
+/* TreeBuilder::UpdatePositions (build_tree.cu:1026-1080): every pair of a node that split moves to
+ * the child its row falls into (X[row][feature[node]] <= split[node] goes left), the others retire
+ * (node -1); then the stable sort by node. `positions` is updated in place; its pairs are of
+ * `level` or retired. */
+size_t lbt_update_positions_workspace_bytes(int64_t n_rows, int32_t level);
+int lbt_update_positions(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                         int32_t* positions, const int32_t* feature, const double* split, int32_t level,
+                         void* workspace, size_t workspace_bytes);
+
 /* Device scratch for lbt_predict: room for the ensemble packed into one node array and one
  * leaf array (total_nodes = sum of the trees' node counts). Returns 0 for invalid arguments. */
 size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t n_outputs, int32_t x_dtype);

@@ -429,6 +429,36 @@ __global__ void root_leaf_kernel(double* leaf, const I64Pair* node_sums, int K,
 // (feature, node), 64 bins per step
 // ---------------------------------------------------------------------------
 
+// Running sums over the 64 lanes of a wave through the lanes' own data paths (DPP operands)
+// instead of LDS permutes, of which a 64-bit scan by shuffles needs two dozen: inside every row
+// of 16 lanes by shifts of 1, 2, 4 and 8 lanes (a lane without a source reads zero), then the
+// last lane of row 0 into row 1 and of row 2 into row 3, then lane 31 into rows 2 and 3.
+// All 64 lanes must be active.
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int64_t dpp_take(int64_t v)
+{
+  const int lo = __builtin_amdgcn_update_dpp(0, static_cast<int>(static_cast<uint32_t>(v)), kCtrl, kRowMask, 0xf, true);
+  const int hi = __builtin_amdgcn_update_dpp(0, static_cast<int>(v >> 32), kCtrl, kRowMask, 0xf, true);
+  return static_cast<int64_t>((static_cast<uint64_t>(static_cast<uint32_t>(hi)) << 32) | static_cast<uint32_t>(lo));
+}
+__device__ __forceinline__ int64_t wave_inclusive_sum(int64_t v)
+{
+  v += dpp_take<0x111, 0xf>(v);  // row_shr:1
+  v += dpp_take<0x112, 0xf>(v);  // row_shr:2
+  v += dpp_take<0x114, 0xf>(v);  // row_shr:4
+  v += dpp_take<0x118, 0xf>(v);  // row_shr:8
+  v += dpp_take<0x142, 0xa>(v);  // row_bcast:15, rows 1 and 3
+  v += dpp_take<0x143, 0xc>(v);  // row_bcast:31, rows 2 and 3
+  return v;
+}
+// value of lane `src` (the same for the whole wave) in every lane
+__device__ __forceinline__ int64_t wave_read_lane(int64_t v, int src)
+{
+  const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(v)), src));
+  const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v >> 32), src));
+  return static_cast<int64_t>((static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 __global__ void __launch_bounds__(kThreads)
   scan_kernel(HistView hist, const I64Pair* node_sums, int F, const int32_t* row_pointers,
               int node_begin, int n_nodes)
@@ -450,16 +480,8 @@ __global__ void __launch_bounds__(kThreads)
     const int bin  = base + lane;
     const bool in  = bin < fe;
     I64Pair* cell  = hist.at(node, k, in ? bin : fb);
-    int64_t eg = in ? cell->grad : 0, eh = in ? cell->hess : 0;
-    for (int off = 1; off < 64; off <<= 1) {
-      int64_t og = __shfl_up(eg, off, 64);
-      int64_t oh = __shfl_up(eh, off, 64);
-      if (lane >= off) {
-        eg += og;
-        eh += oh;
-      }
-    }
-    int64_t tile_g = __shfl(eg, 63, 64), tile_h = __shfl(eh, 63, 64);
+    int64_t eg = wave_inclusive_sum(in ? cell->grad : 0), eh = wave_inclusive_sum(in ? cell->hess : 0);
+    int64_t tile_g = wave_read_lane(eg, 63), tile_h = wave_read_lane(eh, 63);
     eg += agg_g;
     eh += agg_h;
     // the reference skips the store when the running sum is not positive
@@ -672,18 +694,10 @@ __global__ void __launch_bounds__(kThreads)
       else if (base + 64 < fe)
         fetch(base + 64, 0, ns_next, val_next, other_next);
       if (ns.hess > 0) {
-        int64_t eg = val.grad, eh = val.hess;
-        for (int off = 1; off < 64; off <<= 1) {
-          const int64_t og = __shfl_up(eg, off, 64);
-          const int64_t oh = __shfl_up(eh, off, 64);
-          if (lane >= off) {
-            eg += og;
-            eh += oh;
-          }
-        }
-        const int64_t tile_g = __shfl(eg, 63, 64), tile_h = __shfl(eh, 63, 64);
-        eg += __shfl(agg_g, k, 64);
-        eh += __shfl(agg_h, k, 64);
+        int64_t eg = wave_inclusive_sum(val.grad), eh = wave_inclusive_sum(val.hess);
+        const int64_t tile_g = wave_read_lane(eg, 63), tile_h = wave_read_lane(eh, 63);
+        eg += wave_read_lane(agg_g, k);
+        eh += wave_read_lane(agg_h, k);
         // the reference skips the store when the running sum is not positive
         // (build_tree.cu:645); the raw bin value then stays in place
         if (in && (eg > 0 || eh > 0)) {
@@ -1775,6 +1789,8 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
         hb.j0 = j0; hb.n_nodes = n_nodes; hb.level_first = level_first; hb.proposals = L.proposals;
         hb.row_pointers = L.row_pointers; hb.bin_feature = L.bin_feature; hb.hist = hv; hb.qstats = L.qstats; hb.node_sums = L.node_sums;
         hb.level_total = L.level_totals + depth; hb.n_rows = N;
+        // the root's rows are still in their original order, and its launch fills the bin cache first
+        hb.fill_cache = depth == 0; hb.identity = depth == 0;
         LBT_TRY(hist_launch(stream, hs, hb, depth));
       }
       // One pass that scans and evaluates reads the histograms once instead of twice and saves a
@@ -2207,6 +2223,484 @@ int lbt_quantise_gradients_static(void* stream, const double* g, const double* h
   lbt::zero_kernel<<<1, lbt::kThreads, 0, s>>>(reinterpret_cast<uint4*>(root_sums), n_outputs);
   return lbt::run_quantiser(s, g, h, n_rows, n_outputs, row_offset, seed, w.part_a, w.part_b, scales, w.qstats,
                             reinterpret_cast<int2*>(quantised), reinterpret_cast<lbt::I64Pair*>(root_sums));
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------
+// The level's stages on the reference's own layouts: the histogram as
+// [node - first node of the buffer][output][bin] of (int64 grad, int64 hess)
+// (build_tree.h:231-306), the row positions as (node, row) pairs sorted by node
+// with the retired rows (node -1) in front (build_tree.cu:997-1001, :1026-1080).
+// They run the kernels of lbt_build_tree; what is converted on the way in and
+// out is the order (pairs <-> row numbers plus segment starts).
+// ---------------------------------------------------------------------------
+namespace lbt {
+namespace {
+
+// rows[i] = row of pair i
+__global__ void __launch_bounds__(kThreads) pairs_to_rows_kernel(const int2* __restrict__ pairs, int64_t n, int32_t* rows)
+{
+  const int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (i < n) rows[i] = pairs[i].y;
+}
+
+// seg[j] = first pair whose node is >= level_first + j, j = 0 .. n_nodes (the pairs ascend by node)
+__global__ void __launch_bounds__(kThreads)
+  segment_starts_kernel(const int2* __restrict__ pairs, int64_t n, int level_first, int n_nodes, int32_t* seg)
+{
+  const int64_t j = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (j > n_nodes) return;
+  const int64_t want = static_cast<int64_t>(level_first) + j;
+  int64_t lo = 0, hi = n;
+  while (lo < hi) {
+    const int64_t mid = lo + ((hi - lo) >> 1);
+    if (pairs[mid].x < want)
+      lo = mid + 1;
+    else
+      hi = mid;
+  }
+  seg[j] = static_cast<int32_t>(lo);
+}
+
+// block_seg[b] = segment that holds index b * kPartBlock (-1: a retired row); of several segments
+// that start at the same index the last one
+__global__ void __launch_bounds__(kThreads)
+  slab_segments_kernel(const int32_t* __restrict__ seg, int n_nodes, int64_t n_slabs, int32_t* block_seg)
+{
+  const int64_t b = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (b >= n_slabs) return;
+  const int64_t i = b * kPartBlock;
+  int lo = 0, hi = n_nodes;  // number of starts seg[0 .. n_nodes) that are <= i
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (seg[mid] <= i)
+      lo = mid + 1;
+    else
+      hi = mid;
+  }
+  block_seg[b] = lo - 1;
+}
+
+// every pair that is not of the level (or retired): flag[0] = 1
+__global__ void __launch_bounds__(kThreads)
+  check_level_kernel(const int2* __restrict__ pairs, int64_t n, int level_first, int level_end, int64_t n_rows,
+                     int32_t* flag)
+{
+  const int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (i >= n) return;
+  const int2 p  = pairs[i];
+  const bool ok = (p.x == -1 || (p.x >= level_first && p.x < level_end)) && p.y >= 0 && p.y < n_rows &&
+                  (i == 0 || pairs[i - 1].x <= p.x);
+  if (!ok) *flag = 1;
+}
+
+__global__ void __launch_bounds__(kThreads) bin_feature_kernel(const int32_t* row_pointers, int32_t* bin_feature)
+{
+  const int f = blockIdx.x;
+  for (int b = row_pointers[f] + threadIdx.x; b < row_pointers[f + 1]; b += kThreads) bin_feature[b] = f;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads) widen_kernel(const T* in, int64_t n, double* out)
+{
+  const int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x;
+  if (i < n) out[i] = static_cast<double>(in[i]);
+}
+
+// qstats[0] = max |q| over all 2 * n quantised values (qstats cleared by the caller)
+__global__ void __launch_bounds__(kThreads) max_abs_kernel(const int32_t* q, int64_t n2, unsigned long long* qstats)
+{
+  unsigned long long mx = 0;
+  const int64_t stride  = static_cast<int64_t>(gridDim.x) * kThreads;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(kThreads) + threadIdx.x; i < n2; i += stride) {
+    const int64_t v              = q[i];
+    const unsigned long long a   = static_cast<unsigned long long>(v < 0 ? -v : v);
+    mx                           = a > mx ? a : mx;
+  }
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned long long o = __shfl_down(mx, off, 64);
+    mx                         = o > mx ? o : mx;
+  }
+  if ((threadIdx.x & 63) == 0 && mx != 0) atomicMax(&qstats[0], mx);
+}
+
+struct HistStageLayout {
+  // independent of the level, so that the bin cache of one call is where the next call looks for it
+  int32_t* groups;
+  int32_t* sgroups;
+  int64_t* bin_base;
+  int32_t* bin_stride;
+  int32_t* bin_tail;
+  RecInfo* rec;
+  void* upload_block;
+  size_t upload_bytes;
+  void* binned;
+  size_t binned_bytes;
+  uint32_t* tables;
+  void* cell_lo;
+  void* cell_invw;
+  int32_t* bin_feature;
+  unsigned long long* qstats;
+  int32_t* flag;
+  int32_t* rows;
+  int4* tiles;
+  LevelMeta* meta;
+  LevelMeta* level_total;
+  int32_t* pair_sync;
+  unsigned long long* partials;
+  int32_t* partial_lists;
+  int32_t* partial_list_count;
+  int32_t* partial_count;
+  // sized by the level
+  int32_t* seg;
+  int32_t* tile_start;
+};
+
+void make_hist_stage_layout(Arena& ar, HistStageLayout& L, int64_t N, int F, int S, size_t elem, int level)
+{
+  const int64_t level_nodes = int64_t(1) << level;
+  const size_t upload_at    = ar.used;
+  L.groups       = ar.take<int32_t>(F + 1);
+  L.sgroups      = ar.take<int32_t>(F + 1);
+  L.bin_base     = ar.take<int64_t>(F);
+  L.bin_stride   = ar.take<int32_t>(F);
+  L.bin_tail     = ar.take<int32_t>(F);
+  L.rec          = ar.take<RecInfo>(F);
+  L.upload_block = L.groups;
+  L.upload_bytes = ar.used - upload_at;
+  L.binned_bytes = static_cast<size_t>(N) * bin_row_bytes_max(F, S);
+  L.binned       = ar.take<char>(L.binned_bytes + 16);
+  L.tables       = ar.take<uint32_t>(static_cast<size_t>(F) * kMaxCells / 16);
+  L.cell_lo      = ar.take<double>(F);
+  L.cell_invw    = ar.take<double>(F);
+  L.bin_feature  = ar.take<int32_t>(static_cast<size_t>(F) * S);
+  L.qstats       = ar.take<unsigned long long>(2);
+  L.flag         = ar.take<int32_t>(4);
+  L.rows         = ar.take<int32_t>(N);
+  L.tiles        = ar.take<int4>(N / 8 + level_nodes + 1);
+  L.meta         = ar.take<LevelMeta>(1);
+  L.level_total  = ar.take<LevelMeta>(1);
+  L.pair_sync    = ar.take<int32_t>(kPairSyncSlots);
+  L.partials     = ar.take<unsigned long long>(static_cast<size_t>(kPartialSlots) * kPartialStrideMax);
+  L.partial_lists      = ar.take<int32_t>(static_cast<size_t>(kPartialMaxLists) * kPartialListCap);
+  L.partial_list_count = ar.take<int32_t>(kPartialMaxLists);
+  L.partial_count      = ar.take<int32_t>(1);
+  L.seg        = ar.take<int32_t>(level_nodes + 1);
+  L.tile_start = ar.take<int32_t>(level_nodes + 1);
+}
+
+struct SplitStageLayout {
+  int32_t* bin_feature;  // [bins]
+  double* proposals_d;   // [bins]
+  int32_t* split_bin;    // [batch_end]
+  Cand* partial;         // [nodes of the batch][max(chunks, features)]
+};
+
+void make_split_stage_layout(Arena& ar, SplitStageLayout& L, int F, int B, int batch_begin, int batch_end)
+{
+  const int64_t n_chunks = std::max<int64_t>((static_cast<int64_t>(B) + kSplitChunk - 1) / kSplitChunk, F);
+  L.bin_feature = ar.take<int32_t>(B);
+  L.proposals_d = ar.take<double>(B);
+  L.split_bin   = ar.take<int32_t>(batch_end);
+  L.partial     = ar.take<Cand>(static_cast<int64_t>(batch_end - batch_begin) * n_chunks);
+}
+
+struct PositionStageLayout {
+  int32_t* rows[2];
+  int32_t* seg[2];
+  int32_t* block_seg[2];
+  uint8_t* code;
+  int2* block_counts;
+  int2* block_offsets;
+  int2* totals;
+  int2* seg_prefix;
+  int32_t* flag;
+};
+
+void make_position_stage_layout(Arena& ar, PositionStageLayout& L, int64_t N, int level)
+{
+  const int64_t parents = int64_t(1) << level;
+  const int64_t slabs   = (N + kPartBlock - 1) / kPartBlock;
+  for (int i = 0; i < 2; i++) {
+    L.rows[i]      = ar.take<int32_t>(N);
+    L.seg[i]       = ar.take<int32_t>(2 * parents + 1);
+    L.block_seg[i] = ar.take<int32_t>(slabs);
+  }
+  L.code          = ar.take<uint8_t>(N);
+  L.block_counts  = ar.take<int2>(slabs);
+  L.block_offsets = ar.take<int2>(slabs);
+  L.totals        = ar.take<int2>(1);
+  L.seg_prefix    = ar.take<int2>(parents);
+  L.flag          = ar.take<int32_t>(4);
+}
+
+int stage_batch_ok(int32_t level, int32_t batch_begin, int32_t batch_end)
+{
+  LBT_REQUIRE(level >= 0 && level <= 24, "level %d out of range [0,24]", level);
+  LBT_REQUIRE(batch_begin >= level_begin(level) && batch_end <= level_end(level) && batch_begin < batch_end,
+              "nodes [%d, %d) are not a batch of level %d", batch_begin, batch_end, level);
+  return LBT_OK;
+}
+
+int level_of_node(int node)
+{
+  int l = 0;
+  while (level_end(l) <= node) l++;
+  return l;
+}
+
+}  // namespace
+}  // namespace lbt
+
+extern "C" {
+
+size_t lbt_histogram_level_workspace_bytes(int64_t n_rows, int32_t n_features, int32_t split_samples, int32_t x_dtype,
+                                           int32_t level)
+{
+  if (n_rows < 1 || n_rows >= 2147483647LL || n_features < 1 || level < 0 || level > 24) return 0;
+  if (split_samples < 1 || split_samples > LBT_MAX_SPLIT_SAMPLES) return 0;
+  if (x_dtype != LBT_F32 && x_dtype != LBT_F64) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  lbt::HistStageLayout L{};
+  lbt::make_hist_stage_layout(ar, L, n_rows, n_features, split_samples, x_dtype == LBT_F64 ? 8 : 4, level);
+  return ar.used + 256;
+}
+
+int lbt_histogram_level(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                        const int32_t* quantised, int32_t n_outputs, const void* proposals,
+                        const int32_t* row_pointers, int32_t split_samples, const int32_t* positions, int32_t level,
+                        int32_t batch_begin, int32_t batch_end, const int64_t* node_sums, int32_t hist_node_begin,
+                        int32_t hist_node_end, int64_t* histogram, void* workspace, size_t workspace_bytes,
+                        int32_t reuse_bins)
+{
+  using namespace lbt;
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(n_rows >= 1 && n_rows < 2147483647LL && n_features >= 1 && n_outputs >= 1 && n_outputs <= 65535,
+              "bad shape");
+  LBT_REQUIRE(split_samples >= 1 && split_samples <= LBT_MAX_SPLIT_SAMPLES, "split_samples must be in [1, %d]",
+              LBT_MAX_SPLIT_SAMPLES);
+  LBT_REQUIRE(X && quantised && proposals && row_pointers && positions && node_sums && histogram,
+              "null input or output pointer");
+  LBT_TRY(stage_batch_ok(level, batch_begin, batch_end));
+  LBT_REQUIRE(hist_node_begin <= batch_begin && batch_end <= hist_node_end,
+              "the histogram buffer [%d, %d) does not hold the batch [%d, %d)", hist_node_begin, hist_node_end,
+              batch_begin, batch_end);
+  Arena ar;
+  LBT_TRY(arena_over(ar, workspace, workspace_bytes));
+  HistStageLayout L{};
+  const size_t elem = x_dtype == LBT_F64 ? 8 : 4;
+  make_hist_stage_layout(ar, L, n_rows, n_features, split_samples, elem, level);
+  if (ar.failed) {
+    set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto blocks   = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+  const int F = n_features, K = n_outputs;
+  const int64_t N = n_rows;
+  // the bin counts decide the kernels' layout: the one host wait of this call
+  std::vector<int32_t> rp(F + 1);
+  LBT_HIP(hipMemcpyAsync(rp.data(), row_pointers, sizeof(int32_t) * (F + 1), hipMemcpyDeviceToHost, s));
+  LBT_HIP(hipStreamSynchronize(s));
+  LBT_REQUIRE(rp[0] == 0, "row_pointers[0] must be 0");
+  for (int f = 0; f < F; f++)
+    LBT_REQUIRE(rp[f + 1] > rp[f] && rp[f + 1] - rp[f] <= split_samples,
+                "feature %d has %d proposals (1 to split_samples = %d expected)", f, rp[f + 1] - rp[f], split_samples);
+  const int B = rp[F];
+
+  const int level_first = static_cast<int>(level_begin(level));
+  const int level_nodes = 1 << level;
+  const int2* pairs     = reinterpret_cast<const int2*>(positions);
+  {
+    ProfScope ps(LBT_PROF_OTHER, s);
+    zero_kernel<<<1, kThreads, 0, s>>>(reinterpret_cast<uint4*>(L.qstats), 1);
+    zero_kernel<<<1, kThreads, 0, s>>>(reinterpret_cast<uint4*>(L.flag), 1);
+    zero_kernel<<<1, kThreads, 0, s>>>(reinterpret_cast<uint4*>(L.level_total), 2);
+    check_level_kernel<<<blocks(N, kThreads), kThreads, 0, s>>>(pairs, N, level_first, level_first + level_nodes, N, L.flag);
+    pairs_to_rows_kernel<<<blocks(N, kThreads), kThreads, 0, s>>>(pairs, N, L.rows);
+    segment_starts_kernel<<<blocks(level_nodes + 1, kThreads), kThreads, 0, s>>>(pairs, N, level_first, level_nodes, L.seg);
+    max_abs_kernel<<<std::min<unsigned>(blocks(N * K * 2, kThreads), 2048u), kThreads, 0, s>>>(quantised, N * K * 2,
+                                                                                              L.qstats);
+    if (!reuse_bins) bin_feature_kernel<<<F, kThreads, 0, s>>>(row_pointers, L.bin_feature);
+  }
+  int32_t bad = 0;
+  LBT_HIP(hipMemcpyAsync(&bad, L.flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  LBT_HIP(hipStreamSynchronize(s));
+  LBT_REQUIRE(bad == 0, "positions must be (node, row) pairs sorted by node whose nodes are -1 or of level %d", level);
+
+  HistSetup hs;
+  hs.groups = L.groups; hs.sgroups = L.sgroups; hs.tables = L.tables; hs.cell_lo = L.cell_lo; hs.cell_invw = L.cell_invw;
+  hs.tile_start = L.tile_start; hs.tiles = L.tiles; hs.binned = L.binned; hs.binned_capacity = L.binned_bytes;
+  hs.bin_base = L.bin_base; hs.bin_stride = L.bin_stride; hs.bin_tail = L.bin_tail; hs.rec = L.rec;
+  hs.upload_block = L.upload_block; hs.upload_bytes = L.upload_bytes;
+  hs.bins_t = nullptr;  // the feature-major copy serves the position updates of a whole build only
+  hs.bins_t_stride = 0;
+  hs.meta = L.meta; hs.pair_sync = L.pair_sync; hs.partials = L.partials; hs.partial_lists = L.partial_lists;
+  hs.partial_list_count = L.partial_list_count; hs.partial_count = L.partial_count; hs.partial_slots = kPartialSlots;
+  // the tables are built again on every call (they are small); the cache itself is what reuse_bins keeps
+  LBT_TRY(hist_prepare(s, hs, x_dtype == LBT_F64, F, K, N, rp, proposals, row_pointers, X));
+
+  HistBatch hb;
+  hb.X = X; hb.F = F; hb.qgh = reinterpret_cast<const int2*>(quantised); hb.K = K; hb.rows = L.rows; hb.seg = L.seg;
+  hb.j0 = batch_begin - level_first; hb.n_nodes = batch_end - batch_begin; hb.level_first = level_first;
+  hb.proposals = proposals; hb.row_pointers = row_pointers; hb.bin_feature = L.bin_feature;
+  hb.hist = HistView{reinterpret_cast<I64Pair*>(histogram), hist_node_begin, hist_node_end, K, B};
+  hb.qstats = L.qstats; hb.node_sums = reinterpret_cast<const I64Pair*>(node_sums); hb.level_total = L.level_total;
+  hb.n_rows = N; hb.fill_cache = !reuse_bins; hb.identity = false;
+  LBT_TRY(hist_launch(s, hs, hb, level));
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
+int lbt_scan(void* stream, int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end, int32_t n_outputs,
+             int32_t n_features, const int32_t* row_pointers, int32_t n_bins, const int64_t* node_sums,
+             int32_t batch_begin, int32_t batch_end)
+{
+  using namespace lbt;
+  LBT_REQUIRE(histogram && row_pointers && node_sums, "null input or output pointer");
+  LBT_REQUIRE(n_features >= 1 && n_outputs >= 1 && n_outputs <= 65535 && n_bins >= n_features, "bad shape");
+  LBT_TRY(stage_batch_ok(level_of_node(batch_begin), batch_begin, batch_end));
+  LBT_REQUIRE(hist_node_begin <= batch_begin && batch_end <= hist_node_end,
+              "the histogram buffer [%d, %d) does not hold the batch [%d, %d)", hist_node_begin, hist_node_end,
+              batch_begin, batch_end);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  ProfScope ps(LBT_PROF_SCAN, s);
+  const HistView hv{reinterpret_cast<I64Pair*>(histogram), hist_node_begin, hist_node_end, n_outputs, n_bins};
+  const int n_nodes   = batch_end - batch_begin;
+  const int64_t waves = static_cast<int64_t>(n_features) * n_nodes;
+  dim3 grid(static_cast<unsigned>((waves + kThreads / 64 - 1) / (kThreads / 64)), n_outputs);
+  scan_kernel<<<grid, kThreads, 0, s>>>(hv, reinterpret_cast<const I64Pair*>(node_sums), n_features, row_pointers,
+                                        batch_begin, n_nodes);
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
+size_t lbt_best_split_workspace_bytes(int32_t n_features, int32_t n_bins, int32_t batch_begin, int32_t batch_end)
+{
+  if (n_features < 1 || n_bins < n_features || batch_begin < 0 || batch_end <= batch_begin) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  lbt::SplitStageLayout L{};
+  lbt::make_split_stage_layout(ar, L, n_features, n_bins, batch_begin, batch_end);
+  return ar.used + 256;
+}
+
+int lbt_best_split(void* stream, const int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end,
+                   int32_t n_outputs, int32_t n_features, const void* proposals, int32_t x_dtype,
+                   const int32_t* row_pointers, int32_t n_bins, const uint8_t* feature_set, int64_t* node_sums,
+                   const double* scales, double l1_regularization, double l2_regularization, double min_split_gain,
+                   int32_t batch_begin, int32_t batch_end, double* leaf, int32_t* feature, double* split, double* gain,
+                   void* workspace, size_t workspace_bytes)
+{
+  using namespace lbt;
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(histogram && proposals && row_pointers && node_sums && scales && leaf && feature && split && gain,
+              "null input or output pointer");
+  LBT_REQUIRE(n_features >= 1 && n_outputs >= 1 && n_outputs <= 65535 && n_bins >= n_features, "bad shape");
+  LBT_TRY(stage_batch_ok(level_of_node(batch_begin), batch_begin, batch_end));
+  LBT_REQUIRE(hist_node_begin <= batch_begin && batch_end <= hist_node_end,
+              "the histogram buffer [%d, %d) does not hold the batch [%d, %d)", hist_node_begin, hist_node_end,
+              batch_begin, batch_end);
+  Arena ar;
+  LBT_TRY(arena_over(ar, workspace, workspace_bytes));
+  SplitStageLayout L{};
+  make_split_stage_layout(ar, L, n_features, n_bins, batch_begin, batch_end);
+  if (ar.failed) {
+    set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto blocks   = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+  ProfScope ps(LBT_PROF_SPLIT, s);
+  bin_feature_kernel<<<n_features, kThreads, 0, s>>>(row_pointers, L.bin_feature);
+  if (x_dtype == LBT_F64)
+    widen_kernel<double><<<blocks(n_bins, kThreads), kThreads, 0, s>>>(static_cast<const double*>(proposals), n_bins,
+                                                                      L.proposals_d);
+  else
+    widen_kernel<float><<<blocks(n_bins, kThreads), kThreads, 0, s>>>(static_cast<const float*>(proposals), n_bins,
+                                                                     L.proposals_d);
+  // the histogram is only read here; HistView carries it as a mutable pointer for the kernels that fill it
+  const HistView hv{reinterpret_cast<I64Pair*>(const_cast<int64_t*>(histogram)), hist_node_begin, hist_node_end,
+                    n_outputs, n_bins};
+  const int n_nodes  = batch_end - batch_begin;
+  const int n_chunks = (n_bins + kSplitChunk - 1) / kSplitChunk;
+  dim3 grid(n_nodes, n_chunks);
+  split_eval_kernel<<<grid, kThreads, 0, s>>>(hv, reinterpret_cast<const I64Pair*>(node_sums), L.bin_feature,
+                                              feature_set, scales, l1_regularization, l2_regularization,
+                                              min_split_gain, batch_begin, n_chunks, L.partial);
+  split_apply_kernel<<<n_nodes, 64, 0, s>>>(hv, reinterpret_cast<I64Pair*>(node_sums), L.bin_feature, L.proposals_d,
+                                            scales, l1_regularization, l2_regularization, batch_begin, n_chunks,
+                                            L.partial, leaf, feature, split, gain, row_pointers, L.split_bin, true);
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
+}
+
+size_t lbt_update_positions_workspace_bytes(int64_t n_rows, int32_t level)
+{
+  if (n_rows < 1 || n_rows >= 2147483647LL || level < 0 || level > 23) return 0;
+  lbt::Arena ar;
+  ar.measure = true;
+  lbt::PositionStageLayout L{};
+  lbt::make_position_stage_layout(ar, L, n_rows, level);
+  return ar.used + 256;
+}
+
+int lbt_update_positions(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
+                         int32_t* positions, const int32_t* feature, const double* split, int32_t level,
+                         void* workspace, size_t workspace_bytes)
+{
+  using namespace lbt;
+  LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
+  LBT_REQUIRE(n_rows >= 1 && n_rows < 2147483647LL && n_features >= 1, "bad shape");
+  LBT_REQUIRE(level >= 0 && level <= 23, "level %d out of range [0,23]", level);
+  LBT_REQUIRE(X && positions && feature && split, "null input or output pointer");
+  Arena ar;
+  LBT_TRY(arena_over(ar, workspace, workspace_bytes));
+  PositionStageLayout L{};
+  make_position_stage_layout(ar, L, n_rows, level);
+  if (ar.failed) {
+    set_error("workspace too small: %zu bytes given, %zu needed", workspace_bytes, ar.used + 256);
+    return LBT_ERR_WORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto blocks   = [](int64_t n, int t) { return static_cast<unsigned>((n + t - 1) / t); };
+  const int64_t N       = n_rows;
+  const int level_first = static_cast<int>(level_begin(level));
+  const int n_parents   = 1 << level;
+  const unsigned nb     = blocks(N, kPartBlock);
+  int2* pairs           = reinterpret_cast<int2*>(positions);
+  {
+    ProfScope ps(LBT_PROF_OTHER, s);
+    zero_kernel<<<1, kThreads, 0, s>>>(reinterpret_cast<uint4*>(L.flag), 1);
+    check_level_kernel<<<blocks(N, kThreads), kThreads, 0, s>>>(pairs, N, level_first, level_first + n_parents, N, L.flag);
+    pairs_to_rows_kernel<<<blocks(N, kThreads), kThreads, 0, s>>>(pairs, N, L.rows[0]);
+    segment_starts_kernel<<<blocks(n_parents + 1, kThreads), kThreads, 0, s>>>(pairs, N, level_first, n_parents, L.seg[0]);
+    slab_segments_kernel<<<blocks(nb, kThreads), kThreads, 0, s>>>(L.seg[0], n_parents, nb, L.block_seg[0]);
+  }
+  int32_t bad = 0;
+  LBT_HIP(hipMemcpyAsync(&bad, L.flag, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  LBT_HIP(hipStreamSynchronize(s));
+  LBT_REQUIRE(bad == 0, "positions must be (node, row) pairs sorted by node whose nodes are -1 or of level %d", level);
+  ProfScope ps(LBT_PROF_POSITIONS, s);
+  if (x_dtype == LBT_F64)
+    classify_kernel<double><<<nb, kThreads, 0, s>>>(L.rows[0], N, L.seg[0], L.block_seg[0], n_parents, level_first,
+                                                    static_cast<const double*>(X), n_features, feature, split, L.code,
+                                                    L.block_counts);
+  else
+    classify_kernel<float><<<nb, kThreads, 0, s>>>(L.rows[0], N, L.seg[0], L.block_seg[0], n_parents, level_first,
+                                                   static_cast<const float*>(X), n_features, feature, split, L.code,
+                                                   L.block_counts);
+  scan_block_counts_kernel<<<1, kScanThreads, 0, s>>>(L.block_counts, nb, L.block_offsets, L.totals);
+  child_segments_kernel<<<blocks(static_cast<int64_t>(n_parents) * 64, kThreads), kThreads, 0, s>>>(
+    L.seg[0], n_parents, N, L.code, L.block_offsets, L.totals, L.seg_prefix, L.seg[1], L.block_seg[1]);
+  scatter_kernel<<<nb, kThreads, 0, s>>>(L.rows[0], N, L.code, L.block_offsets, L.seg[0], L.block_seg[0], L.seg_prefix,
+                                         L.seg[1], level_first, n_parents, L.rows[1], nullptr);
+  expand_positions_kernel<<<nb, kThreads, 0, s>>>(L.rows[1], N, L.seg[1], L.block_seg[1], 2 * n_parents,
+                                                  static_cast<int>(level_begin(level + 1)), pairs);
+  LBT_HIP(hipGetLastError());
+  return LBT_OK;
 }
 
 int lbt_build_tree(void* stream, const void* X, int32_t x_dtype, int64_t row_offset,

@@ -1525,7 +1525,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   int device = 0, n_cu = 256;
   LBT_HIP(hipGetDevice(&device));
   LBT_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, device));
-  if (use_cache && depth == 0) {
+  if (use_cache && b.fill_cache) {
     // fill the bin cache: rows split evenly over as many workgroups as are resident at once
     // X read once, one bin written per value; with embedded gradients also one pair read and
     // one written per row and histogram group
@@ -1569,7 +1569,7 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     LBT_TRY(rc);
   }
   // the root launch on cached bins also writes the feature-major copy (four rows per lane and tile)
-  const bool root = use_cache && depth == 0 && hs.bins_t != nullptr;
+  const bool root = use_cache && b.identity && hs.bins_t != nullptr;
   TileWalk w;
   unsigned grid = 0;
   LBT_TRY(fill_walk(w, b, n_cu, hs.n_groups, use_cache ? hs.brpp : hs.rpp,
@@ -1639,10 +1639,10 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
   a.search_steps = hs.search_steps;
   a.hist         = b.hist;
   if (hs.vec == 4) {
-    if constexpr (sizeof(T) == 4) return launch_search_rows<T, 4>(stream, hs, a, b, grid, depth == 0);
+    if constexpr (sizeof(T) == 4) return launch_search_rows<T, 4>(stream, hs, a, b, grid, b.identity);
   }
-  if (hs.vec == 2) return launch_search_rows<T, 2>(stream, hs, a, b, grid, depth == 0);
-  return launch_search_rows<T, 1>(stream, hs, a, b, grid, depth == 0);
+  if (hs.vec == 2) return launch_search_rows<T, 2>(stream, hs, a, b, grid, b.identity);
+  return launch_search_rows<T, 1>(stream, hs, a, b, grid, b.identity);
 }
 
 // Packs consecutive features, `unit` at a time, into groups whose LDS need

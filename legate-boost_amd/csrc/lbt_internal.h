@@ -428,6 +428,8 @@ struct HistBatch {
   const I64Pair* node_sums;
   LevelMeta* level_total;
   int64_t n_rows;
+  bool fill_cache;  // run the binning pass first (the bin cache does not hold this X and these proposals yet)
+  bool identity;    // rows[i] == i for every i (the root of a tree that starts from the original order)
 };
 
 // Chooses groups / table size from the host copy of the row pointers and builds

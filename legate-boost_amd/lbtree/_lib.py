@@ -155,6 +155,27 @@ def _load():
     lib.lbt_quantise_gradients_static.restype = C.c_int
     lib.lbt_quantise_gradients_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64,
                                                   C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.lbt_histogram_level_workspace_bytes.restype = C.c_size_t
+    lib.lbt_histogram_level_workspace_bytes.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.lbt_histogram_level.restype = C.c_int
+    lib.lbt_histogram_level.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_int32,
+                                        C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
+                                        C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int32]
+    lib.lbt_scan.restype = C.c_int
+    lib.lbt_scan.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int32,
+                             C.c_void_p, C.c_int32, C.c_int32]
+    lib.lbt_best_split_workspace_bytes.restype = C.c_size_t
+    lib.lbt_best_split_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    lib.lbt_best_split.restype = C.c_int
+    lib.lbt_best_split.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p,
+                                   C.c_int32, C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
+                                   C.c_double, C.c_double, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
+                                   C.c_void_p, C.c_void_p, C.c_size_t]
+    lib.lbt_update_positions_workspace_bytes.restype = C.c_size_t
+    lib.lbt_update_positions_workspace_bytes.argtypes = [C.c_int64, C.c_int32]
+    lib.lbt_update_positions.restype = C.c_int
+    lib.lbt_update_positions.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p,
+                                         C.c_void_p, C.c_int32, C.c_void_p, C.c_size_t]
     lib.lbt_profile_enable.restype = None
     lib.lbt_profile_enable.argtypes = [C.c_int]
     lib.lbt_profile_reset.restype = None
@@ -171,7 +192,10 @@ EXPORTS = [
     "lbt_update_tree_workspace_bytes", "lbt_update_tree", "lbt_weighted_gradient", "lbt_weighted_gradient_sums",
     "lbt_abs_sum_chunks", "lbt_add_leaf_values",
     "lbt_gather_rows", "lbt_select_split_samples_workspace_bytes", "lbt_select_split_samples",
-    "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_quantise_gradients_static", "lbt_profile_enable", "lbt_profile_reset",
+    "lbt_quantise_gradients_workspace_bytes", "lbt_quantise_gradients", "lbt_quantise_gradients_static",
+    "lbt_histogram_level_workspace_bytes", "lbt_histogram_level", "lbt_scan", "lbt_best_split_workspace_bytes",
+    "lbt_best_split", "lbt_update_positions_workspace_bytes", "lbt_update_positions",
+    "lbt_profile_enable", "lbt_profile_reset",
     "lbt_profile_get",
 ]
 

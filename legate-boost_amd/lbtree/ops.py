@@ -371,3 +371,76 @@ def quantise_gradients(g, h, seed, row_offset=0):
                                          sums.data_ptr(), scales.data_ptr(), ws.data_ptr(), ws.numel())
     _lib.check(rc)
     return q, sums, scales
+
+
+# ---- the stages of one level on the reference's layouts (include/lbtree.h) -----------------------
+
+def _stage_ws(nbytes, device):
+    return torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+
+
+def histogram_level(X, quantised, proposals, row_pointers, split_samples, positions, level, batch, node_sums,
+                    hist_nodes, histogram, workspace=None, reuse_bins=False, deepest_level=None):
+    """HistogramKernel of one batch (build_tree.cu:213-577): adds to `histogram`
+    [hist_nodes[1] - hist_nodes[0]][K][n_bins][2] int64. Returns the workspace, which holds the
+    cached bins for a later call with reuse_bins=True; a workspace allocated here is sized for
+    levels up to deepest_level (the part that depends on the level lies behind the cache)."""
+    X = _check_x(X)
+    n, f = X.shape
+    k = quantised.shape[1]
+    dt = _DT[X.dtype]
+    need = _lib.lib.lbt_histogram_level_workspace_bytes(n, f, split_samples, dt, level)
+    if workspace is None:
+        need = max(need, _lib.lib.lbt_histogram_level_workspace_bytes(n, f, split_samples, dt,
+                                                                      max(level, deepest_level or 0)))
+    if workspace is None or workspace.numel() < need:
+        if reuse_bins:
+            raise _lib.LbtError("reuse_bins needs the workspace of the call that cached the bins")
+        workspace = _stage_ws(need, X.device)
+    rc = _lib.lib.lbt_histogram_level(_stream(), X.data_ptr(), dt, n, f, quantised.data_ptr(), k, proposals.data_ptr(),
+                                      row_pointers.data_ptr(), split_samples, positions.data_ptr(), level, batch[0],
+                                      batch[1], node_sums.data_ptr(), hist_nodes[0], hist_nodes[1],
+                                      histogram.data_ptr(), workspace.data_ptr(), workspace.numel(), int(reuse_bins))
+    _lib.check(rc)
+    return workspace
+
+
+def scan(histogram, hist_nodes, row_pointers, n_bins, node_sums, batch):
+    """scan_kernel of one batch (build_tree.cu:597-668), in place."""
+    k = histogram.shape[1]
+    f = row_pointers.numel() - 1
+    rc = _lib.lib.lbt_scan(_stream(), histogram.data_ptr(), hist_nodes[0], hist_nodes[1], k, f, row_pointers.data_ptr(),
+                           n_bins, node_sums.data_ptr(), batch[0], batch[1])
+    _lib.check(rc)
+
+
+def best_split(histogram, hist_nodes, proposals, row_pointers, n_bins, node_sums, scales, batch, leaf, feature, split,
+               gain, l1_regularization=0.0, l2_regularization=1.0, min_split_gain=0.0, feature_set=None):
+    """perform_best_split of one batch (build_tree.cu:682-782): updates node_sums, leaf, feature,
+    split and gain in place."""
+    k = histogram.shape[1]
+    f = row_pointers.numel() - 1
+    ws = _stage_ws(_lib.lib.lbt_best_split_workspace_bytes(f, n_bins, batch[0], batch[1]), histogram.device)
+    fs = None
+    if feature_set is not None:
+        fs = as_device(np.asarray(feature_set, dtype=np.uint8) if not isinstance(feature_set, torch.Tensor)
+                       else feature_set.to(torch.uint8))
+    rc = _lib.lib.lbt_best_split(_stream(), histogram.data_ptr(), hist_nodes[0], hist_nodes[1], k, f,
+                                 proposals.data_ptr(), _DT[proposals.dtype], row_pointers.data_ptr(), n_bins,
+                                 fs.data_ptr() if fs is not None else None, node_sums.data_ptr(), scales.data_ptr(),
+                                 l1_regularization, l2_regularization, min_split_gain, batch[0], batch[1],
+                                 leaf.data_ptr(), feature.data_ptr(), split.data_ptr(), gain.data_ptr(), ws.data_ptr(),
+                                 ws.numel())
+    _lib.check(rc)
+    torch.cuda.current_stream().synchronize()  # ws and fs are released when this returns
+
+
+def update_positions(X, positions, feature, split, level):
+    """UpdatePositions (build_tree.cu:1026-1080), in place on the (node, row) pairs."""
+    X = _check_x(X)
+    n, f = X.shape
+    ws = _stage_ws(_lib.lib.lbt_update_positions_workspace_bytes(n, level), X.device)
+    rc = _lib.lib.lbt_update_positions(_stream(), X.data_ptr(), _DT[X.dtype], n, f, positions.data_ptr(),
+                                       feature.data_ptr(), split.data_ptr(), level, ws.data_ptr(), ws.numel())
+    _lib.check(rc)
+    torch.cuda.current_stream().synchronize()

@@ -406,6 +406,233 @@ static void stable_sort_positions(int32_t* pos, int64_t n, int32_t max_nodes)
   free(count);
 }
 
+/* ------------------------------------------------------------------------- */
+/* The stages of one level. orc_build_tree below is these four in a loop; they   */
+/* are exported so that the library's stage entry points have a twin each.      */
+/* ------------------------------------------------------------------------- */
+
+/* HistogramKernel / fill_histogram_shared, build_tree.cu:332-441 and :445-577: every
+ * instance of the batch whose node is built adds its quantised pair to the bin of each of
+ * its feature values. Integer sums, so the shared/global tile distinction of the kernel
+ * has no effect on the result. bins (optional): bins[row * F + f] = find_bin of that value,
+ * which the reference recomputes at every level (:349, :397). counts (optional): instances
+ * in the batch, instances of built nodes, built nodes that hold rows are added to counts[0..2]. */
+static void histogram_level(const void* X, int is64, int64_t N, int32_t F, const int64_t* q, int32_t K,
+                            const double* proposals, const int32_t* rp, const int32_t* bins, const int32_t* pos,
+                            int batch_begin, int batch_end, int whole_level, const int64_t* node_sums, orc_hist* hs,
+                            int64_t* counts)
+{
+  /* PrepareBatches, build_tree.cu:1207-1258: a level that is one batch takes every instance
+   * (:1212-1216); else lower_bound on node >= batch_begin, upper_bound on node <= batch_end - 1 */
+  int64_t inst_lo = 0, inst_hi = N;
+  if (!whole_level) {
+    int64_t lo = 0, hi = N;
+    while (lo < hi) {
+      int64_t mid = lo + (hi - lo) / 2;
+      if (pos[2 * mid] < batch_begin) lo = mid + 1; else hi = mid;
+    }
+    inst_lo = lo;
+    hi      = N;
+    while (lo < hi) {
+      int64_t mid = lo + (hi - lo) / 2;
+      if (!(batch_end - 1 < pos[2 * mid])) lo = mid + 1; else hi = mid;
+    }
+    inst_hi = lo;
+  }
+  int last_built_node   = -1;
+  if (counts) counts[0] += inst_hi - inst_lo;
+  for (int64_t i = inst_lo; i < inst_hi; i++) {
+    int node = pos[2 * i], row = pos[2 * i + 1];
+    if (node < batch_begin || node >= batch_end) continue; /* a whole level also walks the retired rows */
+    if (!compute_histogram_bin(node, node_sums, K, hist_contains_node(hs, parent_of(node)))) continue;
+    if (counts) counts[1]++;
+    /* the order is sorted by node: a node that is built and holds rows is counted at its first row */
+    if (node != last_built_node) {
+      if (counts) counts[2]++;
+      last_built_node = node;
+    }
+    for (int f = 0; f < F; f++) {
+      int b = bins ? bins[(int64_t)row * F + f] : find_bin(proposals, rp, f, get_x(X, is64, (int64_t)row * F + f));
+      for (int k = 0; k < K; k++) {
+        int64_t* c = hist_at(hs, node, k, b);
+        c[0] += q[((int64_t)row * K + k) * 2 + 0];
+        c[1] += q[((int64_t)row * K + k) * 2 + 1];
+      }
+    }
+  }
+}
+
+/* scan_kernel, build_tree.cu:597-668 */
+static void scan_level(orc_hist* hs, int32_t F, const int32_t* rp, const int64_t* node_sums, int batch_begin,
+                       int batch_end)
+{
+  const int K = hs->K;
+  for (int node = batch_begin; node < batch_end; node++) {
+    int par   = parent_of(node);
+    int built = compute_histogram_bin(node, node_sums, K, hist_contains_node(hs, par));
+    for (int k = 0; k < K; k++) {
+      if (node_sums[((int64_t)node * K + k) * 2 + 1] <= 0) continue;
+      if (!built) continue;
+      for (int f = 0; f < F; f++) {
+        int64_t ag = 0, ah = 0;
+        for (int b = rp[f]; b < rp[f + 1]; b++) {
+          int64_t* c = hist_at(hs, node, k, b);
+          ag += c[0];
+          ah += c[1];
+          /* "Skip write if data is 0", build_tree.cu:645 */
+          if (ag > 0 || ah > 0) {
+            c[0] = ag;
+            c[1] = ah;
+          }
+        }
+        if (node == 0) continue;
+        int sib = sibling_of(node);
+        if (!compute_histogram_bin(sib, node_sums, K, hist_contains_node(hs, par))) {
+          for (int b = rp[f]; b < rp[f + 1]; b++) {
+            int64_t* c  = hist_at(hs, node, k, b);
+            int64_t* pp = hist_at(hs, par, k, b);
+            int64_t* s  = hist_at(hs, sib, k, b);
+            s[0]        = pp[0] - c[0];
+            s[1]        = pp[1] - c[1];
+          }
+        }
+      }
+    }
+  }
+}
+
+/* perform_best_split, build_tree.cu:682-782 */
+static void best_split_level(const orc_hist* hs, int32_t F, const double* proposals, const int32_t* rp,
+                             const uint8_t* feature_set, int64_t* node_sums, const double* scales, double l1,
+                             double l2, double msg, int batch_begin, int batch_end, double* leaf, int32_t* feature,
+                             double* split, double* gain)
+{
+  const int K = hs->K, B = hs->B;
+  for (int node = batch_begin; node < batch_end; node++) {
+    if (node_sums[((int64_t)node * K + 0) * 2 + 1] <= 0) continue;
+    enum { THREADS = 512 };
+    double tg[THREADS];
+    int tb[THREADS];
+    for (int t = 0; t < THREADS; t++) {
+      tg[t] = 0;
+      tb[t] = -1;
+      for (int b = t; b < B; b += THREADS) {
+        if (feature_set && !feature_set[find_feature(rp, F, b)]) continue;
+        double gn = 0;
+        for (int k = 0; k < K; k++) {
+          int64_t ng = node_sums[((int64_t)node * K + k) * 2 + 0];
+          int64_t nh = node_sums[((int64_t)node * K + k) * 2 + 1];
+          int64_t* c = hist_at(hs, node, k, b);
+          int64_t lg = c[0], lh = c[1];
+          int64_t rg = ng - lg, rh = nh - lh;
+          if (lh <= 0 || rh <= 0) {
+            gn = 0;
+            break;
+          }
+          gn += orc_calculate_gain((double)lg * scales[2], (double)lh * scales[3],
+                                   (double)rg * scales[2], (double)rh * scales[3],
+                                   (double)ng * scales[2], (double)nh * scales[3], l1, l2, msg);
+        }
+        if (gn > tg[t]) {
+          tg[t] = gn;
+          tb[t] = b;
+        }
+      }
+    }
+    /* cub::BlockReduce keeps rank order; op(a,b) = a.gain > b.gain ? a : b */
+    double bg = tg[0];
+    int bb    = tb[0];
+    for (int t = 1; t < THREADS; t++) {
+      if (!(bg > tg[t])) {
+        bg = tg[t];
+        bb = tb[t];
+      }
+    }
+    if (bg > 1e-5) {
+      int bf = find_feature(rp, F, bb);
+      for (int k = 0; k < K; k++) {
+        int64_t ng = node_sums[((int64_t)node * K + k) * 2 + 0];
+        int64_t nh = node_sums[((int64_t)node * K + k) * 2 + 1];
+        int64_t* c = hist_at(hs, node, k, bb);
+        int64_t lg = c[0], lh = c[1], rg = ng - lg, rh = nh - lh;
+        int lc = left_child(node), rc = right_child(node);
+        node_sums[((int64_t)lc * K + k) * 2 + 0] = lg;
+        node_sums[((int64_t)lc * K + k) * 2 + 1] = lh;
+        node_sums[((int64_t)rc * K + k) * 2 + 0] = rg;
+        node_sums[((int64_t)rc * K + k) * 2 + 1] = rh;
+        leaf[(int64_t)lc * K + k] = orc_calculate_leaf_value((double)lg * scales[2], (double)lh * scales[3], l1, l2);
+        leaf[(int64_t)rc * K + k] = orc_calculate_leaf_value((double)rg * scales[2], (double)rh * scales[3], l1, l2);
+      }
+      feature[node] = bf;
+      split[node]   = proposals[bb];
+      gain[node]    = bg;
+    }
+  }
+}
+
+/* UpdatePositions, build_tree.cu:1026-1080 */
+static void update_positions(const void* X, int is64, int64_t N, int32_t F, int32_t* pos, const int32_t* feature,
+                             const double* split, int32_t max_nodes)
+{
+  for (int64_t i = 0; i < N; i++) {
+    int ps = pos[2 * i], row = pos[2 * i + 1];
+    if (ps < 0 || ps >= max_nodes || feature[ps] == -1) {
+      pos[2 * i] = -1;
+      continue;
+    }
+    double xv  = get_x(X, is64, (int64_t)row * F + feature[ps]);
+    pos[2 * i] = xv <= split[ps] ? left_child(ps) : right_child(ps);
+  }
+  stable_sort_positions(pos, N, max_nodes);
+}
+
+static double* proposals_as_double(const void* proposals, int is64, int32_t B)
+{
+  double* p = (double*)malloc(sizeof(double) * (size_t)(B > 0 ? B : 1));
+  for (int i = 0; i < B; i++) p[i] = is64 ? ((const double*)proposals)[i] : (double)((const float*)proposals)[i];
+  return p;
+}
+
+void orc_histogram_level(const void* X, int is64, int64_t N, int32_t F, const int64_t* q, int32_t K,
+                         const void* proposals, const int32_t* rp, const int32_t* pos, int32_t batch_begin,
+                         int32_t batch_end, const int64_t* node_sums, int32_t hist_node_begin,
+                         int32_t hist_node_end, int64_t* histogram)
+{
+  double* pd = proposals_as_double(proposals, is64, rp[F]);
+  orc_hist hs;
+  hs.data = histogram; hs.node_begin = hist_node_begin; hs.node_end = hist_node_end; hs.K = K; hs.B = rp[F];
+  histogram_level(X, is64, N, F, q, K, pd, rp, NULL, pos, batch_begin, batch_end, 0, node_sums, &hs, NULL);
+  free(pd);
+}
+
+void orc_scan(int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end, int32_t K, int32_t F,
+              const int32_t* rp, const int64_t* node_sums, int32_t batch_begin, int32_t batch_end)
+{
+  orc_hist hs;
+  hs.data = histogram; hs.node_begin = hist_node_begin; hs.node_end = hist_node_end; hs.K = K; hs.B = rp[F];
+  scan_level(&hs, F, rp, node_sums, batch_begin, batch_end);
+}
+
+void orc_best_split(const int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end, int32_t K, int32_t F,
+                    const void* proposals, int is64, const int32_t* rp, const uint8_t* feature_set,
+                    int64_t* node_sums, const double scales[4], double l1, double l2, double min_split_gain,
+                    int32_t batch_begin, int32_t batch_end, double* leaf, int32_t* feature, double* split,
+                    double* gain)
+{
+  double* pd = proposals_as_double(proposals, is64, rp[F]);
+  orc_hist hs;
+  hs.data = (int64_t*)histogram; hs.node_begin = hist_node_begin; hs.node_end = hist_node_end; hs.K = K; hs.B = rp[F];
+  best_split_level(&hs, F, pd, rp, feature_set, node_sums, scales, l1, l2, min_split_gain, batch_begin, batch_end,
+                   leaf, feature, split, gain);
+  free(pd);
+}
+
+void orc_update_positions(const void* X, int is64, int64_t N, int32_t F, int32_t* pos, const int32_t* feature,
+                          const double* split, int32_t max_nodes)
+{
+  update_positions(X, is64, N, F, pos, feature, split, max_nodes);
+}
+
 int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32_t F,
                    const double* g, const double* h, int32_t K, const uint8_t* feature_set,
                    const orc_params* p, double* leaf, int32_t* feature, double* split,
@@ -486,9 +713,7 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
   for (int depth = 0; depth < max_depth; depth++) {
     if (taps && taps->positions_per_level)
       memcpy(taps->positions_per_level + (size_t)depth * N * 2, pos, sizeof(int32_t) * 2 * (size_t)N);
-    int64_t lvl_inst = 0, lvl_built_inst = 0;
-    int32_t lvl_built_nodes = 0;
-    int last_built_node     = -1;
+    int64_t counts[3] = {0, 0, 0};
 
     /* PrepareBatches, build_tree.cu:1207-1258 */
     const int64_t nodes_in_level = (int64_t)1 << depth;
@@ -497,29 +722,13 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
       num_batches = (nodes_in_level + max_batch_size - 1) / max_batch_size;
     for (int64_t bi = 0; bi < num_batches; bi++) {
       int batch_begin, batch_end;
-      int64_t inst_lo, inst_hi;
       if (num_batches == 1) {
         batch_begin = (int)level_begin(depth);
         batch_end   = (int)level_end(depth);
-        inst_lo     = 0;
-        inst_hi     = N;
       } else {
         batch_begin = (int)(level_begin(depth) + bi * max_batch_size);
         int64_t e   = (int64_t)batch_begin + max_batch_size;
         batch_end   = (int)(e < level_end(depth) ? e : level_end(depth));
-        /* lower_bound on node >= batch_begin; upper_bound on node <= batch_end-1 */
-        int64_t lo = 0, hi = N;
-        while (lo < hi) {
-          int64_t mid = lo + (hi - lo) / 2;
-          if (pos[2 * mid] < batch_begin) lo = mid + 1; else hi = mid;
-        }
-        inst_lo = lo;
-        hi      = N;
-        while (lo < hi) {
-          int64_t mid = lo + (hi - lo) / 2;
-          if (!(batch_end - 1 < pos[2 * mid])) lo = mid + 1; else hi = mid;
-        }
-        inst_hi = lo;
       }
 
       /* GetHistogram, build_tree.cu:1191-1205 */
@@ -530,142 +739,17 @@ int orc_build_tree(const void* X, int is64, int64_t row_offset, int64_t N, int32
         hs.data = (int64_t*)calloc((size_t)(batch_end - batch_begin) * K * B * 2, sizeof(int64_t));
       }
 
-      /* fill_histogram_shared, build_tree.cu:332-441: integer sums, so the
-       * shared/global tile distinction has no effect on the result. */
-      lvl_inst += inst_hi - inst_lo;
-      for (int64_t i = inst_lo; i < inst_hi; i++) {
-        int node = pos[2 * i], row = pos[2 * i + 1];
-        if (!compute_histogram_bin(node, node_sums, K, hist_contains_node(&hs, parent_of(node))))
-          continue;
-        lvl_built_inst++;
-        /* the order is sorted by node: a node that is built and holds rows is counted at its first row */
-        if (node != last_built_node) {
-          lvl_built_nodes++;
-          last_built_node = node;
-        }
-        for (int f = 0; f < F; f++) {
-          int b = bins[(int64_t)row * F + f];
-          for (int k = 0; k < K; k++) {
-            int64_t* c = hist_at(&hs, node, k, b);
-            c[0] += q[((int64_t)row * K + k) * 2 + 0];
-            c[1] += q[((int64_t)row * K + k) * 2 + 1];
-          }
-        }
-      }
-
-      /* scan_kernel, build_tree.cu:597-668 */
-      for (int node = batch_begin; node < batch_end; node++) {
-        int par = parent_of(node);
-        int built = compute_histogram_bin(node, node_sums, K, hist_contains_node(&hs, par));
-        for (int k = 0; k < K; k++) {
-          if (node_sums[((int64_t)node * K + k) * 2 + 1] <= 0) continue;
-          if (!built) continue;
-          for (int f = 0; f < F; f++) {
-            int64_t ag = 0, ah = 0;
-            for (int b = rp[f]; b < rp[f + 1]; b++) {
-              int64_t* c = hist_at(&hs, node, k, b);
-              ag += c[0];
-              ah += c[1];
-              /* "Skip write if data is 0", build_tree.cu:645 */
-              if (ag > 0 || ah > 0) {
-                c[0] = ag;
-                c[1] = ah;
-              }
-            }
-            if (node == 0) continue;
-            int sib = sibling_of(node);
-            if (!compute_histogram_bin(sib, node_sums, K, hist_contains_node(&hs, par))) {
-              for (int b = rp[f]; b < rp[f + 1]; b++) {
-                int64_t* c  = hist_at(&hs, node, k, b);
-                int64_t* pp = hist_at(&hs, par, k, b);
-                int64_t* s  = hist_at(&hs, sib, k, b);
-                s[0]        = pp[0] - c[0];
-                s[1]        = pp[1] - c[1];
-              }
-            }
-          }
-        }
-      }
-
-      /* perform_best_split, build_tree.cu:682-782 */
-      for (int node = batch_begin; node < batch_end; node++) {
-        if (node_sums[((int64_t)node * K + 0) * 2 + 1] <= 0) continue;
-        enum { THREADS = 512 };
-        double tg[THREADS];
-        int tb[THREADS];
-        for (int t = 0; t < THREADS; t++) {
-          tg[t] = 0;
-          tb[t] = -1;
-          for (int b = t; b < B; b += THREADS) {
-            if (feature_set && !feature_set[find_feature(rp, F, b)]) continue;
-            double gn = 0;
-            for (int k = 0; k < K; k++) {
-              int64_t ng = node_sums[((int64_t)node * K + k) * 2 + 0];
-              int64_t nh = node_sums[((int64_t)node * K + k) * 2 + 1];
-              int64_t* c = hist_at(&hs, node, k, b);
-              int64_t lg = c[0], lh = c[1];
-              int64_t rg = ng - lg, rh = nh - lh;
-              if (lh <= 0 || rh <= 0) {
-                gn = 0;
-                break;
-              }
-              gn += orc_calculate_gain((double)lg * scales[2], (double)lh * scales[3],
-                                       (double)rg * scales[2], (double)rh * scales[3],
-                                       (double)ng * scales[2], (double)nh * scales[3], l1, l2, msg);
-            }
-            if (gn > tg[t]) {
-              tg[t] = gn;
-              tb[t] = b;
-            }
-          }
-        }
-        /* cub::BlockReduce keeps rank order; op(a,b) = a.gain > b.gain ? a : b */
-        double bg = tg[0];
-        int bb    = tb[0];
-        for (int t = 1; t < THREADS; t++) {
-          if (!(bg > tg[t])) {
-            bg = tg[t];
-            bb = tb[t];
-          }
-        }
-        if (bg > 1e-5) {
-          int bf = find_feature(rp, F, bb);
-          for (int k = 0; k < K; k++) {
-            int64_t ng = node_sums[((int64_t)node * K + k) * 2 + 0];
-            int64_t nh = node_sums[((int64_t)node * K + k) * 2 + 1];
-            int64_t* c = hist_at(&hs, node, k, bb);
-            int64_t lg = c[0], lh = c[1], rg = ng - lg, rh = nh - lh;
-            int lc = left_child(node), rc = right_child(node);
-            node_sums[((int64_t)lc * K + k) * 2 + 0] = lg;
-            node_sums[((int64_t)lc * K + k) * 2 + 1] = lh;
-            node_sums[((int64_t)rc * K + k) * 2 + 0] = rg;
-            node_sums[((int64_t)rc * K + k) * 2 + 1] = rh;
-            leaf[(int64_t)lc * K + k] = orc_calculate_leaf_value((double)lg * scales[2], (double)lh * scales[3], l1, l2);
-            leaf[(int64_t)rc * K + k] = orc_calculate_leaf_value((double)rg * scales[2], (double)rh * scales[3], l1, l2);
-          }
-          feature[node] = bf;
-          split[node]   = proposals[bb];
-          gain[node]    = bg;
-        }
-      }
+      histogram_level(X, is64, N, F, q, K, proposals, rp, bins, pos, batch_begin, batch_end, num_batches == 1,
+                      node_sums, &hs, counts);
+      scan_level(&hs, F, rp, node_sums, batch_begin, batch_end);
+      best_split_level(&hs, F, proposals, rp, feature_set, node_sums, scales, l1, l2, msg, batch_begin, batch_end,
+                       leaf, feature, split, gain);
     }
-    if (taps && taps->level_instances) taps->level_instances[depth] = lvl_inst;
-    if (taps && taps->level_built_instances) taps->level_built_instances[depth] = lvl_built_inst;
-    if (taps && taps->level_built_nodes) taps->level_built_nodes[depth] = lvl_built_nodes;
+    if (taps && taps->level_instances) taps->level_instances[depth] = counts[0];
+    if (taps && taps->level_built_instances) taps->level_built_instances[depth] = counts[1];
+    if (taps && taps->level_built_nodes) taps->level_built_nodes[depth] = (int32_t)counts[2];
 
-    /* UpdatePositions, build_tree.cu:1026-1080 */
-    if (depth < max_depth - 1) {
-      for (int64_t i = 0; i < N; i++) {
-        int ps = pos[2 * i], row = pos[2 * i + 1];
-        if (ps < 0 || ps >= max_nodes || feature[ps] == -1) {
-          pos[2 * i] = -1;
-          continue;
-        }
-        double xv  = get_x(X, is64, (int64_t)row * F + feature[ps]);
-        pos[2 * i] = xv <= split[ps] ? left_child(ps) : right_child(ps);
-      }
-      stable_sort_positions(pos, N, max_nodes);
-    }
+    if (depth < max_depth - 1) update_positions(X, is64, N, F, pos, feature, split, max_nodes);
   }
 
   /* WriteTreeOutput, build_tree.cu:826-845 */

@@ -131,6 +131,37 @@ int orc_build_tree(const void* X, int x_is_f64, int64_t row_offset, int64_t n_ro
                    int32_t* feature, double* split, double* gain, double* hessian,
                    orc_taps* taps);
 
+/* ---- the stages of one level on their own (orc_build_tree runs these four in a loop) ---- */
+
+/* HistogramKernel, build_tree.cu:332-577, for the nodes [batch_begin, batch_end) of one level:
+ * quantised [n_rows][K][2] int64, proposals of X's type, positions [n_rows][2] (node, row) sorted
+ * by node; adds to histogram [hist_node_end - hist_node_begin][K][row_pointers[F]][2]. */
+void orc_histogram_level(const void* X, int x_is_f64, int64_t n_rows, int32_t n_features,
+                         const int64_t* quantised, int32_t n_outputs, const void* proposals,
+                         const int32_t* row_pointers, const int32_t* positions, int32_t batch_begin,
+                         int32_t batch_end, const int64_t* node_sums, int32_t hist_node_begin,
+                         int32_t hist_node_end, int64_t* histogram);
+
+/* scan_kernel, build_tree.cu:597-668: running sums per feature, in place, and the siblings
+ * that are not built derived from their parents. */
+void orc_scan(int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end, int32_t n_outputs,
+              int32_t n_features, const int32_t* row_pointers, const int64_t* node_sums,
+              int32_t batch_begin, int32_t batch_end);
+
+/* perform_best_split, build_tree.cu:682-782, on a scanned histogram: writes feature, split and
+ * gain of the nodes that split, and node_sums and leaf of their children. */
+void orc_best_split(const int64_t* histogram, int32_t hist_node_begin, int32_t hist_node_end,
+                    int32_t n_outputs, int32_t n_features, const void* proposals, int x_is_f64,
+                    const int32_t* row_pointers, const uint8_t* feature_set, int64_t* node_sums,
+                    const double scales[4], double l1, double l2, double min_split_gain,
+                    int32_t batch_begin, int32_t batch_end, double* leaf, int32_t* feature,
+                    double* split, double* gain);
+
+/* UpdatePositions, build_tree.cu:1026-1080: positions [n_rows][2] in place. */
+void orc_update_positions(const void* X, int x_is_f64, int64_t n_rows, int32_t n_features,
+                          int32_t* positions, const int32_t* feature, const double* split,
+                          int32_t max_nodes);
+
 /* predict.cu:26-84. Trees are given as arrays of pointers. out[n_rows*K]. */
 void orc_predict(const void* X, int x_is_f64, int64_t n_rows, int32_t n_features,
                  int32_t n_trees, const double* const* leaf, const int32_t* const* feature,

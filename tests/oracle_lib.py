@@ -103,6 +103,20 @@ def _load():
     lib.orc_gather_rows.restype = None
     lib.orc_gather_rows.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_int64,
                                     C.c_void_p]
+    lib.orc_histogram_level.restype = None
+    lib.orc_histogram_level.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p,
+                                        C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_int32, C.c_int32,
+                                        C.c_void_p]
+    lib.orc_scan.restype = None
+    lib.orc_scan.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32,
+                             C.c_int32]
+    lib.orc_best_split.restype = None
+    lib.orc_best_split.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_int,
+                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_double, C.c_double,
+                                   C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    lib.orc_update_positions.restype = None
+    lib.orc_update_positions.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p,
+                                         C.c_int32]
     return lib
 
 
@@ -304,3 +318,38 @@ def gather_rows(X, rows, row_offset=0):
     out = np.empty((rows.shape[0], X.shape[1]), X.dtype)
     lib.orc_gather_rows(_p(X), is64, row_offset, X.shape[0], X.shape[1], _p(rows), rows.shape[0], _p(out))
     return out
+
+
+# ---- the stages of one level (orc_build_tree runs these four in a loop); arrays are updated in place
+
+def histogram_level(X, quantised, proposals, row_pointers, positions, batch, node_sums, hist_nodes, histogram):
+    X, is64 = _check_x(X)
+    n, f = X.shape
+    assert quantised.dtype == np.int64 and positions.dtype == np.int32 and histogram.dtype == np.int64
+    assert proposals.dtype == X.dtype and node_sums.dtype == np.int64 and row_pointers.dtype == np.int32
+    lib.orc_histogram_level(_p(X), is64, n, f, _p(quantised), quantised.shape[1], _p(proposals), _p(row_pointers),
+                            _p(positions), batch[0], batch[1], _p(node_sums), hist_nodes[0], hist_nodes[1],
+                            _p(histogram))
+
+
+def scan(histogram, hist_nodes, row_pointers, node_sums, batch):
+    assert histogram.dtype == np.int64 and node_sums.dtype == np.int64
+    lib.orc_scan(_p(histogram), hist_nodes[0], hist_nodes[1], histogram.shape[1], len(row_pointers) - 1,
+                 _p(row_pointers), _p(node_sums), batch[0], batch[1])
+
+
+def best_split(histogram, hist_nodes, proposals, row_pointers, node_sums, scales4, batch, leaf, feature, split, gain,
+               l1=0.0, l2=1.0, min_split_gain=0.0, feature_set=None):
+    fs = None if feature_set is None else np.ascontiguousarray(feature_set, np.uint8)
+    scales4 = np.ascontiguousarray(scales4, np.float64)
+    lib.orc_best_split(_p(histogram), hist_nodes[0], hist_nodes[1], histogram.shape[1], len(row_pointers) - 1,
+                       _p(proposals), int(proposals.dtype == np.float64), _p(row_pointers),
+                       _p(fs) if fs is not None else None, _p(node_sums), _p(scales4), l1, l2, min_split_gain,
+                       batch[0], batch[1], _p(leaf), _p(feature), _p(split), _p(gain))
+
+
+def update_positions(X, positions, feature, split, max_nodes):
+    X, is64 = _check_x(X)
+    n, f = X.shape
+    assert positions.dtype == np.int32 and feature.dtype == np.int32 and split.dtype == np.float64
+    lib.orc_update_positions(_p(X), is64, n, f, _p(positions), _p(feature), _p(split), max_nodes)

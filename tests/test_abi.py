@@ -103,6 +103,29 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert qg(None, one, one, 10, 1, 0, 1, one, one, one, one, 8) == -3
     with pytest.raises(_lib.LbtError):
         _lib.check(rc)
+    # the stages of a level
+    hw = _lib.lib.lbt_histogram_level_workspace_bytes
+    assert 0 < hw(1000, 4, 16, _lib.LBT_F32, 0) < hw(1000, 4, 16, _lib.LBT_F32, 12)
+    assert hw(1000, 4, 4096, _lib.LBT_F32, 0) == 0 and hw(0, 4, 16, _lib.LBT_F32, 0) == 0
+    hl = _lib.lib.lbt_histogram_level
+    assert hl(None, one, _lib.LBT_F32, 10, 2, one, 1, one, one, 16, one, 1, 0, 1, one, 0, 3, one, one, 1 << 20, 0) == -1
+    assert b"not a batch of level" in _lib.lib.lbt_last_error()
+    assert hl(None, one, _lib.LBT_F32, 10, 2, one, 1, one, one, 16, one, 1, 1, 3, one, 2, 3, one, one, 1 << 20, 0) == -1
+    assert b"does not hold the batch" in _lib.lib.lbt_last_error()
+    assert hl(None, one, _lib.LBT_F32, 10, 2, one, 1, one, one, 16, one, 0, 0, 1, one, 0, 1, one, one, 8, 0) == -3
+    assert _lib.lib.lbt_scan(None, one, 0, 3, 1, 2, one, 32, one, 1, 4) == -1
+    assert _lib.lib.lbt_scan(None, None, 0, 3, 1, 2, one, 32, one, 1, 3) == -1
+    assert _lib.lib.lbt_best_split_workspace_bytes(2, 32, 1, 3) > 0
+    assert _lib.lib.lbt_best_split_workspace_bytes(2, 1, 1, 3) == 0
+    bs = _lib.lib.lbt_best_split
+    assert bs(None, one, 0, 3, 1, 2, one, _lib.LBT_F32, one, 32, None, one, one, 0.0, 1.0, 0.0, 1, 3, one, one, one, one,
+              one, 8) == -3
+    assert bs(None, one, 0, 3, 1, 2, one, 9, one, 32, None, one, one, 0.0, 1.0, 0.0, 1, 3, one, one, one, one, one,
+              1 << 20) == -1
+    assert _lib.lib.lbt_update_positions_workspace_bytes(1000, 3) > 0
+    assert _lib.lib.lbt_update_positions_workspace_bytes(1000, 30) == 0
+    assert _lib.lib.lbt_update_positions(None, one, _lib.LBT_F32, 10, 2, None, one, one, 0, one, 1 << 20) == -1
+    assert _lib.lib.lbt_update_positions(None, one, _lib.LBT_F32, 10, 2, one, one, one, 0, one, 8) == -3
 
 
 def test_tree_constructor_mirrors_reference_checks():

@@ -609,3 +609,62 @@ def test_row_leaf_update_equals_predict():
             nd = 2 * nd + 1 if X[r, t.feature[nd]] <= t.split_value[nd] else 2 * nd + 2
         walk[r] = nd
     assert np.array_equal(orc.add_leaf_values(np.zeros((300, 2)), t.leaf_value, walk), pr)
+
+
+def test_the_four_stage_functions_chain_to_the_whole_build():
+    """orc_histogram_level, orc_scan, orc_best_split and orc_update_positions are the loop body of
+    orc_build_tree (pinned above by brute force); driven one by one from Python, with a histogram
+    buffer that is re-allocated for the last level as GetHistogram (build_tree.cu:1191-1205) does,
+    they must give the same tree, histograms and positions."""
+    rs = np.random.RandomState(8)
+    n, f, k, depth, s, seed = 4000, 6, 2, 4, 32, 5
+    X = rs.normal(size=(n, f)).astype(np.float32)
+    g = rs.normal(size=(n, k))
+    h = np.abs(rs.normal(size=(n, k))) + 0.1
+    props, rp = orc.split_proposals(X, seed, s)
+    B = int(rp[-1])
+    cache_nodes = 8  # levels 0..2 share a buffer of 7 nodes, level 3 (8 nodes) gets its own
+    whole = orc.build_tree(X, g, h, max_depth=depth, split_samples=s, seed=seed, hist_cache_bytes=cache_nodes * k * B * 16)
+    assert (whole.hist_node_begin, whole.hist_node_end) == (7, 15)
+    sc = orc.scales(orc.abs_sums(g, h))
+    q = orc.quantise_all(g, h, seed, sc)
+    max_nodes = 2 ** (depth + 1) - 1
+    sums = np.zeros((max_nodes, k, 2), np.int64)
+    sums[0] = q.sum(axis=0)
+    leaf = np.zeros((max_nodes, k))
+    feature = -np.ones(max_nodes, np.int32)
+    split = np.zeros(max_nodes)
+    gain = np.zeros(max_nodes)
+    pos = np.stack([np.zeros(n, np.int32), np.arange(n, dtype=np.int32)], axis=1).copy()
+    hist_nodes = (0, 7)
+    hist = np.zeros((7, k, B, 2), np.int64)
+    for level in range(depth):
+        batch = (2 ** level - 1, 2 ** (level + 1) - 1)
+        if batch[1] > hist_nodes[1]:
+            hist_nodes = batch
+            hist = np.zeros((batch[1] - batch[0], k, B, 2), np.int64)
+        assert np.array_equal(pos, whole.positions_per_level[level]) if whole.positions_per_level is not None else True
+        orc.histogram_level(X, q, props, rp, pos, batch, sums, hist_nodes, hist)
+        orc.scan(hist, hist_nodes, rp, sums, batch)
+        orc.best_split(hist, hist_nodes, props, rp, sums, sc, batch, leaf, feature, split, gain)
+        if level < depth - 1:
+            orc.update_positions(X, pos, feature, split, max_nodes)
+    assert np.array_equal(feature, whole.feature) and (feature != -1).sum() >= 8
+    assert np.array_equal(split, whole.split_value) and np.array_equal(gain, whole.gain)
+    assert np.array_equal(sums, whole.node_sums)
+    assert np.array_equal(leaf[1:], whole.leaf_value[1:])
+    assert np.array_equal(pos, whole.positions)
+    assert np.array_equal(hist, whole.histogram)
+    # a batch that is a part of a level adds the same bins as the level in one piece
+    both = np.zeros((8, k, B, 2), np.int64)
+    orc.histogram_level(X, q, props, rp, pos, (7, 11), sums, (7, 15), both)
+    orc.histogram_level(X, q, props, rp, pos, (11, 15), sums, (7, 15), both)
+    raw = np.zeros((8, k, B, 2), np.int64)
+    orc.histogram_level(X, q, props, rp, pos, (7, 15), sums, (7, 15), raw)
+    assert np.array_equal(both, raw)
+    # every row of every output lands once per feature
+    per_feature = np.add.reduceat(raw, rp[:-1], axis=2)  # [node][k][feature][2]
+    for j in range(8):
+        rows = pos[pos[:, 0] == 7 + j, 1]
+        want = q[rows].sum(axis=0)  # [k][2]
+        assert np.array_equal(per_feature[j], np.repeat(want[:, None, :], f, axis=1))
