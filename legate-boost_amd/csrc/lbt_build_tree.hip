@@ -1797,14 +1797,16 @@ int build_tree_impl(hipStream_t stream, const T* X, int64_t row_offset, int64_t 
       // launch per level. With a single output and many nodes (the deep levels of a deep tree,
       // most of whose nodes are empty or small) the two kernels are faster: the evaluation then
       // runs over all bins of a node side by side, not feature by feature behind the scan.
-      const bool fused = K <= kFusedMaxK && (K >= 2 || n_nodes <= 256);
       // The scanned histograms of this level are read again only by the next level's sibling
       // subtraction (and by a caller that asked to see them): not after the last level, and not
       // when the next level starts a buffer of its own (GetHistogram, build_tree.cu:1191-1205).
       const int64_t next_begin = level_begin(depth + 1), next_end = level_end(depth + 1);
       const bool next_reads    = depth + 1 < max_depth && next_end - next_begin <= max_batch_size &&
                               next_begin >= hv.node_begin && next_end <= hv.node_end;
-      const bool store = !fused || next_reads || (taps && taps->histogram);
+      const bool wanted = next_reads || (taps && taps->histogram);
+      // ... and where nothing reads them again the fused pass, which then only reads, wins as well
+      const bool fused = K <= kFusedMaxK && (K >= 2 || n_nodes <= 256 || !wanted);
+      const bool store = !fused || wanted;
       if (fused) {
         ProfScope ps(LBT_PROF_SCAN, stream);
         const int64_t waves = static_cast<int64_t>(F) * n_nodes;

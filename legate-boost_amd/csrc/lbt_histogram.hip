@@ -153,6 +153,105 @@ __global__ void __launch_bounds__(kPlanThreads)
   tiles[tile]      = make_int4(level_first + j, r0, min(seg_hi, r0 + tile_rows), seg_hi - seg_lo);
 }
 
+// Both of the above in one launch, for batches of up to kPlanFusedNodes nodes: every workgroup
+// repeats the count and the scan of the nodes' tiles (a few loads per thread) instead of waiting
+// for a launch that does it once, then writes the descriptors of its own 256 tiles. Workgroup 0
+// also leaves the batch's totals and clears the counters of the launch that follows.
+constexpr int kPlanFusedNodes = 4096;
+__global__ void __launch_bounds__(kPlanThreads)
+  plan_expand_tiles_kernel(int j0, int j1, int level_first, const int32_t* __restrict__ seg,
+                           const I64Pair* __restrict__ node_sums, int K, int hist_node_begin, int hist_node_end,
+                           int tile_rows, int4* tiles, LevelMeta* meta, LevelMeta* level_total, int32_t* pair_sync,
+                           int32_t* partial_count, int32_t* partial_list_count)
+{
+  __shared__ int s_scan[kPlanThreads];
+  __shared__ unsigned long long s_rb, s_rc, s_nb;
+  const bool first_wg = blockIdx.x == 0;
+  if (first_wg) {
+    if (threadIdx.x == 0) s_rb = s_rc = s_nb = 0;
+    if (pair_sync != nullptr)
+      for (int i = threadIdx.x; i < kPairSyncSlots; i += kPlanThreads) pair_sync[i] = 0;
+    if (partial_count != nullptr) {
+      if (threadIdx.x == 0) *partial_count = 0;
+      for (int i = threadIdx.x; i < kPartialMaxLists; i += kPlanThreads) partial_list_count[i] = 0;
+    }
+  }
+  const int n     = j1 - j0;
+  const int per   = (n + kPlanThreads - 1) / kPlanThreads;
+  const int begin = j0 + min(n, static_cast<int>(threadIdx.x) * per);
+  const int end   = j0 + min(n, (static_cast<int>(threadIdx.x) + 1) * per);
+  auto tiles_of = [&](int j, int& rows, bool& built) {
+    const int node   = level_first + j;
+    rows             = seg[j + 1] - seg[j];
+    const int parent = parent_of(node);
+    const bool pex   = parent >= hist_node_begin && parent < hist_node_end;
+    built            = compute_histogram_bin(node, node_sums, K, pex);
+    return built ? (rows + tile_rows - 1) / tile_rows : 0;
+  };
+  int mine = 0;
+  unsigned long long rb = 0, rc = 0, nb = 0;
+  for (int j = begin; j < end; j++) {
+    int rows;
+    bool built;
+    mine += tiles_of(j, rows, built);
+    rb += static_cast<unsigned long long>(rows);
+    if (built && rows > 0) {
+      rc += static_cast<unsigned long long>(rows);
+      nb += 1;
+    }
+  }
+  s_scan[threadIdx.x] = mine;
+  __syncthreads();
+  for (int off = 1; off < kPlanThreads; off <<= 1) {
+    const int v = static_cast<int>(threadIdx.x) >= off ? s_scan[threadIdx.x - off] : 0;
+    __syncthreads();
+    s_scan[threadIdx.x] += v;
+    __syncthreads();
+  }
+  const int total = s_scan[kPlanThreads - 1];
+  if (first_wg) {
+    if (rb != 0) atomicAdd(&s_rb, rb);
+    if (rc != 0) atomicAdd(&s_rc, rc);
+    if (nb != 0) atomicAdd(&s_nb, nb);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      meta->n_tiles         = total;
+      meta->instances       = s_rb;
+      meta->built_instances = s_rc;
+      meta->built_nodes     = s_nb;
+      level_total->instances += s_rb;
+      level_total->built_instances += s_rc;
+      level_total->built_nodes += s_nb;
+    }
+  }
+  const int tile = blockIdx.x * kPlanThreads + threadIdx.x;
+  if (tile >= total) return;
+  // the thread whose run of nodes holds the tile: the last one whose inclusive count exceeds it
+  int lo = 0, hi = kPlanThreads - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (s_scan[mid] > tile)
+      hi = mid;
+    else
+      lo = mid + 1;
+  }
+  int run       = lo > 0 ? s_scan[lo - 1] : 0;  // first tile of that thread's run
+  const int b2  = j0 + min(n, lo * per);
+  const int e2  = j0 + min(n, (lo + 1) * per);
+  for (int j = b2; j < e2; j++) {
+    int rows;
+    bool built;
+    const int t = tiles_of(j, rows, built);
+    if (tile < run + t) {
+      const int seg_lo = seg[j], seg_hi = seg[j + 1];
+      const int r0     = seg_lo + (tile - run) * tile_rows;
+      tiles[tile]      = make_int4(level_first + j, r0, min(seg_hi, r0 + tile_rows), seg_hi - seg_lo);
+      return;
+    }
+    run += t;
+  }
+}
+
 // The cell of a value, t = x * invw + nlo clamped to [0, cmax]: monotone non-decreasing in x
 // for any nlo and invw >= 0 (a fused multiply-add rounds once, and rounding and clamping keep
 // order); NaN goes to cell 0. Table construction and lookup share this function, which is
@@ -1577,14 +1676,22 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
                     use_cache ? hs.blds_bytes : hs.lds_bytes, &grid));
   {
     ProfScope ps(LBT_PROF_OTHER, stream);
-    plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
-                                                      b.K, b.hist.node_begin, b.hist.node_end, w.tile_rows,
-                                                      hs.tile_start, hs.meta, b.level_total);
     const int64_t max_tiles = (b.n_rows + w.tile_rows - 1) / w.tile_rows + b.n_nodes;
-    expand_tiles_kernel<<<static_cast<unsigned>((max_tiles + kPlanThreads - 1) / kPlanThreads), kPlanThreads, 0,
-                          stream>>>(b.j0, b.n_nodes, b.level_first, b.seg, hs.tile_start, hs.meta, w.tile_rows,
-                                    hs.tiles, root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr,
-                                    use_cache ? hs.partial_count : nullptr, hs.partial_list_count);
+    const unsigned egrid    = static_cast<unsigned>((max_tiles + kPlanThreads - 1) / kPlanThreads);
+    int32_t* const sync     = root && w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr;
+    int32_t* const pcount   = use_cache ? hs.partial_count : nullptr;
+    if (b.n_nodes <= kPlanFusedNodes) {
+      plan_expand_tiles_kernel<<<egrid, kPlanThreads, 0, stream>>>(
+        b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums, b.K, b.hist.node_begin, b.hist.node_end, w.tile_rows,
+        hs.tiles, hs.meta, b.level_total, sync, pcount, hs.partial_list_count);
+    } else {
+      plan_tiles_kernel<<<1, kPlanThreads, 0, stream>>>(b.j0, b.j0 + b.n_nodes, b.level_first, b.seg, b.node_sums,
+                                                        b.K, b.hist.node_begin, b.hist.node_end, w.tile_rows,
+                                                        hs.tile_start, hs.meta, b.level_total);
+      expand_tiles_kernel<<<egrid, kPlanThreads, 0, stream>>>(b.j0, b.n_nodes, b.level_first, b.seg, hs.tile_start,
+                                                              hs.meta, w.tile_rows, hs.tiles, sync, pcount,
+                                                              hs.partial_list_count);
+    }
   }
   if (use_cache) {
     BinnedArgs a;
