@@ -57,6 +57,11 @@ int lbt_release_thread_resources(void);
  * histogram-cache budget that the reference hard-codes to 1e9 bytes
  * (build_tree.cu:1004). hist_cache_bytes == 0 selects that constant. */
 typedef struct lbt_build_params {
+  /* sizeof(lbt_build_params) of the header the caller was built against. The library refuses a
+   * value that is not its own, so a struct of another version of this header, or one that was
+   * never initialised, gives LBT_ERR_INVALID instead of a misread member. Zero-initialise the
+   * struct (lbt_build_params p = {0} / p{}) and set this member first. */
+  int32_t struct_bytes;
   int32_t max_depth;
   int32_t max_nodes; /* must equal 2^(max_depth+1) - 1 */
   int32_t split_samples;
@@ -70,7 +75,8 @@ typedef struct lbt_build_params {
    * writes them for exactly these g and h ([2][lbt_abs_sum_chunks(n_rows, n_outputs)] doubles).
    * With it the build skips its own first pass over g and h for the quantiser's scale
    * (build_tree.cu:77-83); the scale, and with it every result, is the same bit for bit.
-   * NULL: the build sums g and h itself. Sums that belong to other gradients give a wrong scale. */
+   * NULL: the build sums g and h itself. Sums that belong to other gradients give a wrong scale.
+   * The array may not overlap g or h. */
   const double* abs_sum_chunks;
 } lbt_build_params;
 
@@ -203,6 +209,10 @@ int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64
  * All calls on one GPU share that GPU's array: two calls that overlap on one GPU (different
  * streams, or different host threads) race; calls on one stream are ordered. Nothing is
  * carried over from one call to the next.
+ * Under stream capture: make the first call on each device before the capture begins (that call
+ * resolves the array's address, which may load the code object), and leave the profiler off
+ * (lbt_profile_enable(0)): with it on, the call creates and records events. root_sums must be
+ * 16-byte aligned (it is cleared with 16-byte stores by a kernel, not a memset node).
  */
 #define LBT_QUANTISE_STATIC_MAX_ENTRIES (1LL << 26)
 int lbt_quantise_gradients_static(void* stream, const double* g, const double* h, int64_t n_rows,
@@ -289,9 +299,9 @@ size_t lbt_predict_workspace_bytes(int32_t n_trees, int64_t total_nodes, int32_t
  *   workspace           device scratch of at least lbt_predict_workspace_bytes(...), or
  *                       NULL. With it, rows are staged in LDS in tiles of 64 to 256 and walked
  *                       through the packed ensemble batch by batch; without it (or when a
- *                       row tile or a tree does not fit the LDS, or n_outputs > 8) every
- *                       node step reads the trees' own arrays. The sums are the same: a
- *                       row's leaf values are added in tree order either way.
+ *                       row tile or a tree does not fit the LDS) every node step reads the
+ *                       trees' own arrays. More than 8 outputs are walked 8 at a time. The
+ *                       sums are the same: a row's leaf values are added in tree order either way.
  * Work is enqueued on `stream`; the call does not synchronise.
  */
 int lbt_predict(void* stream, const void* X, int32_t x_dtype, int64_t n_rows, int32_t n_features,
@@ -326,8 +336,8 @@ typedef struct lbt_packed_ensemble {
  * Packs n_trees trees (arguments as for lbt_predict) for X of the given dtype and width into
  * `buffer` (device, at least lbt_predict_workspace_bytes(n_trees, total_nodes, n_outputs, x_dtype))
  * and fills *ensemble. The trees' own arrays are not referenced after the stream has passed
- * this call. Returns LBT_ERR_UNSUPPORTED when the shapes do not fit the packed form (more
- * than 8 outputs, a tree of more than 65535 nodes or too large for the LDS, rows too wide):
+ * this call. Returns LBT_ERR_UNSUPPORTED when the shapes do not fit the packed form (a tree
+ * of more than 65535 nodes or too large for the LDS, rows too wide for the LDS):
  * lbt_predict without a workspace serves those.
  */
 int lbt_pack_ensemble(void* stream, int32_t x_dtype, int32_t n_features, int32_t n_trees,

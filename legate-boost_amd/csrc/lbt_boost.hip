@@ -271,6 +271,18 @@ int lbt_weighted_gradient_sums(void* stream, int32_t objective, const double* pr
   hipStream_t s   = static_cast<hipStream_t>(stream);
   const int64_t n = n_rows * n_outputs;
   const int64_t m = lbt_abs_sum_chunks(n_rows, n_outputs);
+  {
+    // the chunk sums are written while the pass still reads pred and y and writes g and h
+    const char* c0 = reinterpret_cast<const char*>(abs_sum_chunks);
+    const char* c1 = c0 + 2 * sizeof(double) * static_cast<size_t>(m);
+    const size_t bytes = sizeof(double) * static_cast<size_t>(n);
+    for (const double* a : {pred, static_cast<const double*>(g), static_cast<const double*>(h)}) {
+      const char* a0 = reinterpret_cast<const char*>(a);
+      LBT_REQUIRE(c1 <= a0 || a0 + bytes <= c0, "abs_sum_chunks may not alias pred, g or h");
+    }
+    const char* y0 = reinterpret_cast<const char*>(y);  // at least n_rows labels
+    LBT_REQUIRE(c1 <= y0 || y0 + sizeof(double) * static_cast<size_t>(n_rows) <= c0, "abs_sum_chunks may not alias y");
+  }
   lbt::ProfScope ps(LBT_PROF_OTHER, s, static_cast<double>(n) * 32.0);
   double* sum_g = abs_sum_chunks;
   double* sum_h = abs_sum_chunks + m;

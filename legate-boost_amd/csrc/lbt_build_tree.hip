@@ -1529,6 +1529,10 @@ void make_layout(Arena& ar, Layout& L, int64_t N, int F, int K, int max_depth, i
 int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
 {
   LBT_REQUIRE(p != nullptr, "params is null");
+  LBT_REQUIRE(p->struct_bytes == static_cast<int32_t>(sizeof(lbt_build_params)),
+              "lbt_build_params.struct_bytes is %d, this library's struct has %d bytes: set it to "
+              "sizeof(lbt_build_params) of the lbtree.h the library was built with, in a zero-initialised struct",
+              p->struct_bytes, static_cast<int>(sizeof(lbt_build_params)));
   LBT_REQUIRE(x_dtype == LBT_F32 || x_dtype == LBT_F64, "unsupported X dtype %d", x_dtype);
   LBT_REQUIRE(N >= 1 && N < 2147483647LL, "n_rows %lld out of range", static_cast<long long>(N));
   LBT_REQUIRE(F >= 1 && K >= 1, "n_features and n_outputs must be positive");
@@ -1549,7 +1553,9 @@ int validate(int64_t N, int F, int K, const lbt_build_params* p, int x_dtype)
 // for by itself and not together with everything else that is queued on the stream.
 int host_mirror(int F, ThreadResources** out)
 {
-  ThreadResources& hm = thread_resources();
+  ThreadResources* here = nullptr;
+  LBT_TRY(thread_resources_here(&here));
+  ThreadResources& hm = *here;
   if (hm.counts_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.counts_here, hipEventDisableTiming));
   if (hm.stats_here == nullptr) LBT_HIP(hipEventCreateWithFlags(&hm.stats_here, hipEventDisableTiming));
   // an earlier call of this thread that did not wait (or failed half-way) may still own the buffer
@@ -2022,6 +2028,7 @@ size_t lbt_build_tree_workspace_bytes(int64_t n_rows, int32_t n_features, int32_
                                       int64_t hist_cache_bytes)
 {
   lbt_build_params p{};
+  p.struct_bytes     = static_cast<int32_t>(sizeof(p));
   p.max_depth        = max_depth;
   p.max_nodes        = max_depth >= 0 && max_depth <= 24 ? static_cast<int32_t>(lbt::level_end(max_depth)) : 0;
   p.split_samples    = split_samples;
@@ -2045,6 +2052,16 @@ static int build_tree_entry(void* stream, const void* X, int32_t x_dtype, int64_
   LBT_TRY(lbt::validate(n_rows, n_features, n_outputs, params, x_dtype));
   LBT_REQUIRE(X && g && h && leaf && feature && split && gain && hessian, "null input or output pointer");
   LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
+  if (params->abs_sum_chunks != nullptr) {
+    // the chunk sums are read while g and h may still be in use by the same pass: no overlap
+    const char* c0 = reinterpret_cast<const char*>(params->abs_sum_chunks);
+    const char* c1 = c0 + 2 * sizeof(double) * static_cast<size_t>((n_rows * n_outputs + 4095) / 4096);
+    const size_t gh_bytes = sizeof(double) * static_cast<size_t>(n_rows) * n_outputs;
+    for (const double* a : {g, h}) {
+      const char* a0 = reinterpret_cast<const char*>(a);
+      LBT_REQUIRE(c1 <= a0 || a0 + gh_bytes <= c0, "abs_sum_chunks overlaps g or h");
+    }
+  }
   if (workspace == nullptr) {
     lbt::set_error("workspace is null; size it with lbt_build_tree_workspace_bytes");
     return LBT_ERR_WORKSPACE;
@@ -2139,6 +2156,7 @@ int lbt_quantise_gradients(void* stream, const double* g, const double* h, int64
   LBT_REQUIRE(n_rows >= 1 && n_rows < 2147483647LL && n_outputs >= 1 && n_outputs <= 65535, "bad shape");
   LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
   LBT_REQUIRE(g && h && quantised && root_sums && scales, "null input or output pointer");
+  LBT_REQUIRE(reinterpret_cast<uintptr_t>(root_sums) % 16 == 0, "root_sums must be 16-byte aligned");
   lbt::Arena ar;
   LBT_TRY(arena_over(ar, workspace, workspace_bytes));
   QuantiserScratch w;
@@ -2206,6 +2224,7 @@ int lbt_quantise_gradients_static(void* stream, const double* g, const double* h
               static_cast<long long>(kStaticMaxEntries), static_cast<long long>(n_rows * static_cast<int64_t>(n_outputs)));
   LBT_REQUIRE(row_offset >= 0, "row_offset must not be negative");
   LBT_REQUIRE(g && h && quantised && root_sums && scales, "null input or output pointer");
+  LBT_REQUIRE(reinterpret_cast<uintptr_t>(root_sums) % 16 == 0, "root_sums must be 16-byte aligned");
   void* scratch = nullptr;
   LBT_TRY(static_scratch_address(&scratch));
   lbt::Arena ar;

@@ -122,29 +122,68 @@ ProfLevels* Profiler::begin_levels(int n_levels, double per_row, double per_node
   return &levels.back();
 }
 
+// Takes the thread's handles out of its record first and then releases every one of them, also
+// after a failure in between: nothing that was freed or destroyed stays reachable for a later
+// call. The first failure is what is reported.
+int release_thread_resources()
+{
+  ThreadResources& tr = thread_resources();
+  const ThreadResources old = tr;
+  tr = ThreadResources{};
+  hipError_t first = hipSuccess;
+  const char* what = "";
+  auto note = [&](hipError_t e, const char* call) {
+    if (e != hipSuccess && first == hipSuccess) {
+      first = e;
+      what  = call;
+    }
+  };
+  // the buffers may still feed or receive copies of calls that did not wait
+  if (old.stage_free != nullptr) note(hipEventSynchronize(old.stage_free), "hipEventSynchronize");
+  if (old.counts_here != nullptr) note(hipEventSynchronize(old.counts_here), "hipEventSynchronize");
+  if (old.stats_here != nullptr) note(hipEventSynchronize(old.stats_here), "hipEventSynchronize");
+  if (old.stage != nullptr) note(hipHostFree(old.stage), "hipHostFree");
+  if (old.mirror != nullptr) note(hipHostFree(old.mirror), "hipHostFree");
+  if (old.stage_free != nullptr) note(hipEventDestroy(old.stage_free), "hipEventDestroy");
+  if (old.counts_here != nullptr) note(hipEventDestroy(old.counts_here), "hipEventDestroy");
+  if (old.stats_here != nullptr) note(hipEventDestroy(old.stats_here), "hipEventDestroy");
+  if (first != hipSuccess) {
+    set_error("%s failed while the thread's resources were released: %s", what, hipGetErrorString(first));
+    return LBT_ERR_HIP;
+  }
+  return LBT_OK;
+}
+
+// The thread's resources for the current device: events and pinned buffers belong to the device
+// they were created on, so a thread that has moved to another device starts afresh.
+int thread_resources_here(ThreadResources** out)
+{
+  int device = 0;
+  LBT_HIP(hipGetDevice(&device));
+  ThreadResources& tr = thread_resources();
+  const bool holds = tr.mirror != nullptr || tr.stage != nullptr || tr.counts_here != nullptr ||
+                     tr.stats_here != nullptr || tr.stage_free != nullptr;
+  if (holds && tr.device != device) {
+    const int now = device;
+    LBT_HIP(hipSetDevice(tr.device));
+    const int rc = release_thread_resources();
+    LBT_HIP(hipSetDevice(now));
+    LBT_TRY(rc);
+  }
+  thread_resources().device = device;
+  *out = &thread_resources();
+  return LBT_OK;
+}
+
 }  // namespace lbt
 
 extern "C" {
 
 const char* lbt_last_error(void) { return lbt::g_error; }
 
-int lbt_version(void) { return 2; }
+int lbt_version(void) { return 3; }
 
-int lbt_release_thread_resources(void)
-{
-  lbt::ThreadResources& tr = lbt::thread_resources();
-  // the buffers may still feed or receive copies of calls that did not wait
-  if (tr.stage_free != nullptr) LBT_HIP(hipEventSynchronize(tr.stage_free));
-  if (tr.counts_here != nullptr) LBT_HIP(hipEventSynchronize(tr.counts_here));
-  if (tr.stats_here != nullptr) LBT_HIP(hipEventSynchronize(tr.stats_here));
-  if (tr.stage != nullptr) LBT_HIP(hipHostFree(tr.stage));
-  if (tr.mirror != nullptr) LBT_HIP(hipHostFree(tr.mirror));
-  if (tr.stage_free != nullptr) LBT_HIP(hipEventDestroy(tr.stage_free));
-  if (tr.counts_here != nullptr) LBT_HIP(hipEventDestroy(tr.counts_here));
-  if (tr.stats_here != nullptr) LBT_HIP(hipEventDestroy(tr.stats_here));
-  tr = lbt::ThreadResources{};
-  return LBT_OK;
-}
+int lbt_release_thread_resources(void) { return lbt::release_thread_resources(); }
 
 void lbt_profile_enable(int on) { lbt::profiler().mode = on < 0 ? 0 : on; }
 

@@ -1841,7 +1841,9 @@ struct Upload {
       const char* d = static_cast<const char*>(it.dst);
       together      = together && d >= lo && d + it.bytes <= lo + block_bytes;
     }
-    ThreadResources& tr = thread_resources();
+    ThreadResources* here = nullptr;
+    LBT_TRY(thread_resources_here(&here));
+    ThreadResources& tr = *here;
     if (together) {
       if (tr.stage_free == nullptr) {
         if (hipEventCreateWithFlags(&tr.stage_free, hipEventDisableTiming) != hipSuccess) together = false;

@@ -132,6 +132,7 @@ struct ProfScope {
 // the thread that calls lbt_build_tree, released by lbt_release_thread_resources() on that
 // thread (or never: a thread that ends without calling it leaves them to the process's end).
 struct ThreadResources {
+  int device = 0;  // the device the handles below were created on
   // what the host reads back in the middle of a build (bin counts per feature, the quantiser's
   // overflow flag): [4 + capacity] ints, two 64-bit statistics first
   int32_t* mirror        = nullptr;
@@ -143,6 +144,9 @@ struct ThreadResources {
   hipEvent_t stage_free = nullptr;
 };
 ThreadResources& thread_resources();
+// the same after making sure that what it holds belongs to the current device
+int thread_resources_here(ThreadResources** out);
+int release_thread_resources();
 
 // ---------------------------------------------------------------- device math
 

@@ -305,33 +305,34 @@ __device__ __forceinline__ void add_in_order(double& run, const double (&val)[S:
 }
 template <typename S, int kAcc, int jj>
 __device__ __forceinline__ void add_leaves_from(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
-                                                const double* __restrict__ batch_leaves, int K)
+                                                const double* __restrict__ batch_leaves, int K, int k0)
 {
   if constexpr (jj < S::kBatchTrees) {
     const int p = from_owner<S, jj>(at);
     if (jj < cnt) {
-      const double* lf = batch_leaves + static_cast<int64_t>(p) * K;
+      const double* lf = batch_leaves + static_cast<int64_t>(p) * K + k0;
 #pragma unroll
       for (int k = 0; k < kAcc; k++)
-        if (k < K) acc[k] += lf[k];
+        if (k0 + k < K) acc[k] += lf[k];
     }
-    add_leaves_from<S, kAcc, jj + 1>(acc, at, cnt, batch_leaves, K);
+    add_leaves_from<S, kAcc, jj + 1>(acc, at, cnt, batch_leaves, K, k0);
   }
 }
 template <typename S, int kAcc>
 __device__ __forceinline__ void add_leaves_in_order(double (&acc)[kAcc], const int (&at)[S::kLaneTrees], int cnt,
-                                                    const double* __restrict__ batch_leaves, int K)
+                                                    const double* __restrict__ batch_leaves, int K, int k0)
 {
-  add_leaves_from<S, kAcc, 0>(acc, at, cnt, batch_leaves, K);
+  add_leaves_from<S, kAcc, 0>(acc, at, cnt, batch_leaves, K, k0);
 }
 
 template <typename T, bool kSingle, int L, bool kFew = false>
 __global__ void __launch_bounds__(kTileThreads)
   predict_tile_kernel(const T* __restrict__ X, int64_t n_rows, int F, int pitch, int n_batches,
                       const BatchInfo* __restrict__ batches, const PackedTree* __restrict__ desc,
-                      const PackedNode<T>* __restrict__ nodes, const double* __restrict__ leaves, int K,
+                      const PackedNode<T>* __restrict__ nodes, const double* __restrict__ leaves, int K, int k0,
                       double* __restrict__ out)
 {
+  // k0: first of the (at most kTileMaxK) outputs this launch sums; more outputs take a launch per chunk
   using S = TileShape<L, kFew>;
   constexpr int kTileRows = S::kRows, kLaneTrees = S::kLaneTrees;
   extern __shared__ __align__(16) unsigned char smem_raw[];  // 16-byte aligned whatever static LDS precedes it
@@ -430,16 +431,16 @@ __global__ void __launch_bounds__(kTileThreads)
       int at[kLaneTrees];
 #pragma unroll
       for (int j = 0; j < kLaneTrees; j++) at[j] = base[j] + pos[j];
-      add_leaves_in_order<S, kAcc>(acc, at, info.count, leaves + info.node_off * K, K);
+      add_leaves_in_order<S, kAcc>(acc, at, info.count, leaves + info.node_off * K, K, k0);
     }
   }
   if constexpr (kSingle) add_in_order<S>(acc[0], val, cnt_prev, q);
   // single output: the row's last lane holds the sum; several outputs: every lane of the row does
   if (valid && q == (kSingle ? L - 1 : 0)) {
-    double* o = out + (row0 + r) * K;
+    double* o = out + (row0 + r) * K + k0;
 #pragma unroll
     for (int k = 0; k < kAcc; k++)
-      if (k < K) o[k] = acc[k];
+      if (k0 + k < K) o[k] = acc[k];
   }
 }
 
@@ -497,7 +498,7 @@ int pack_tiled(hipStream_t stream, int F, int n_trees, const double* const* leaf
                lbt_packed_ensemble* ens)
 {
   *ens = lbt_packed_ensemble{};
-  if (buffer == nullptr || K > kTileMaxK || F > 16383) return LBT_OK;  // a float node holds 4 * feature in 16 bits
+  if (buffer == nullptr || F > 16383) return LBT_OK;  // a float node holds 4 * feature in 16 bits
   int64_t total_nodes = 0;
   int max_nodes       = 0;
   for (int i = 0; i < n_trees; i++) {
@@ -611,10 +612,13 @@ int run_tiled(hipStream_t stream, const T* X, int64_t N, const lbt_packed_ensemb
   const int tile_rows = kTileThreads / lanes;
   ProfScope ps(LBT_PROF_PREDICT, stream, static_cast<double>(N) * (static_cast<double>(F) * sizeof(T) + K * 8.0));
   const unsigned tiles = static_cast<unsigned>((N + tile_rows - 1) / tile_rows);
+  // the kernel sums up to kTileMaxK outputs per walk: more outputs are walked chunk by chunk (each
+  // chunk's sums are formed in tree order, as in one walk)
   auto launch = [&](auto kernel, std::atomic<bool> (&flags)[kMaxDevices]) -> int {
     LBT_TRY(allow_dynamic_lds(kernel, kTileLds, flags));
-    kernel<<<tiles, kTileThreads, static_cast<size_t>(ens.lds_bytes), stream>>>(X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes,
-                                                      lay.leaves, K, out);
+    for (int k0 = 0; k0 < K; k0 += kTileMaxK)
+      kernel<<<tiles, kTileThreads, static_cast<size_t>(ens.lds_bytes), stream>>>(
+        X, N, F, pitch, n_batches, lay.batches, lay.desc, lay.nodes, lay.leaves, K, k0, out);
     return LBT_OK;
   };
   static std::atomic<bool> attr[6][kMaxDevices] = {};
@@ -821,8 +825,8 @@ int lbt_pack_ensemble(void* stream, int32_t x_dtype, int32_t n_features, int32_t
     LBT_TRY(lbt::pack_tiled<double>(s, n_features, n_trees, leaf, feature, split, tree_nodes, n_outputs, buffer,
                                     buffer_bytes, ensemble));
   if (ensemble->data == nullptr) {
-    lbt::set_error("ensemble does not fit the packed form (more than %d outputs, more than 16383 features or "
-                   "nodes per tree, or rows too wide for the LDS): use lbt_predict", lbt::kTileMaxK);
+    lbt::set_error("ensemble does not fit the packed form (more than 16383 features, a tree of more than 65535 "
+                   "nodes or too large for the LDS, or rows too wide for the LDS): use lbt_predict");
     return LBT_ERR_UNSUPPORTED;
   }
   return LBT_OK;
@@ -837,7 +841,7 @@ int lbt_predict_packed(void* stream, const void* X, int32_t x_dtype, int64_t n_r
               n_features, ensemble->x_dtype, ensemble->n_features);
   LBT_REQUIRE((ensemble->lanes == 4 || ensemble->lanes == 8 || ensemble->lanes == 16) && ensemble->n_trees >= 1 &&
                 ensemble->n_batches >= 1 && ensemble->n_batches <= ensemble->n_trees &&
-                ensemble->n_outputs >= 1 && ensemble->n_outputs <= lbt::kTileMaxK &&
+                ensemble->n_outputs >= 1 && ensemble->n_outputs <= 65535 &&
                 ensemble->total_nodes >= ensemble->n_trees && ensemble->lds_bytes >= 16 &&
                 static_cast<size_t>(ensemble->lds_bytes) <= lbt::kTileLds,
               "corrupt ensemble descriptor");

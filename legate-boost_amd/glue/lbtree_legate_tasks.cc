@@ -115,6 +115,7 @@ T* dense_out(legate::PhysicalStore store)
   if (xs.lo[1] != 0) throw std::runtime_error("lbtree: features should not be split between workers");
 
   lbt_build_params p{};
+  p.struct_bytes      = static_cast<int32_t>(sizeof(p));
   p.max_depth         = context.scalars().at(0).value<int>();
   p.max_nodes         = context.scalars().at(1).value<int>();
   p.split_samples     = context.scalars().at(2).value<int>();

@@ -21,7 +21,9 @@ PROF_CLASSES = ["proposals", "quantise", "histogram", "scan", "split", "position
 
 
 class BuildParams(C.Structure):
+    """lbt_build_params; struct_bytes is filled in, the positional arguments start at max_depth."""
     _fields_ = [
+        ("struct_bytes", C.c_int32),
         ("max_depth", C.c_int32),
         ("max_nodes", C.c_int32),
         ("split_samples", C.c_int32),
@@ -33,6 +35,9 @@ class BuildParams(C.Structure):
         ("hist_cache_bytes", C.c_int64),
         ("abs_sum_chunks", C.c_void_p),
     ]
+
+    def __init__(self, *args, **kw):
+        super().__init__(C.sizeof(BuildParams), *args, **kw)
 
 
 class BuildTaps(C.Structure):

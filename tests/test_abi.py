@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(_lib.lib, n), n
     assert sorted(_lib.EXPORTS) == names
-    assert _lib.lib.lbt_version() >= 2
+    assert _lib.lib.lbt_version() >= 3
     assert _lib.lib.lbt_release_thread_resources() == 0  # nothing held yet: nothing to do, no GPU call
 
 
@@ -64,6 +64,16 @@ def test_bad_arguments_are_rejected_without_a_gpu():
                                  one, one, one, 1 << 20, None)
     assert rc == -1 and b"max_nodes" in _lib.lib.lbt_last_error()
     prm.max_nodes = 15
+    prm.struct_bytes = 48  # a struct of another version of the header, or one that was never filled in
+    rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
+                                 one, one, one, 1 << 20, None)
+    assert rc == -1 and b"struct_bytes" in _lib.lib.lbt_last_error()
+    prm.struct_bytes = C.sizeof(_lib.BuildParams)
+    prm.abs_sum_chunks = 16 + 8  # inside g
+    rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
+                                 one, one, one, 1 << 20, None)
+    assert rc == -1 and b"overlaps" in _lib.lib.lbt_last_error()
+    prm.abs_sum_chunks = None
     prm.split_samples = 4096
     rc = _lib.lib.lbt_build_tree(None, one, _lib.LBT_F32, 0, 10, 2, one, one, 1, None, C.byref(prm), one, one, one,
                                  one, one, one, 1 << 20, None)
@@ -101,6 +111,12 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert qg(None, one, one, 10, 0, 0, 1, one, one, one, one, 1 << 20) == -1
     assert qg(None, one, one, 10, 1, 0, 1, one, None, one, one, 1 << 20) == -1
     assert qg(None, one, one, 10, 1, 0, 1, one, one, one, one, 8) == -3
+    assert qg(None, one, one, 10, 1, 0, 1, one, C.c_void_p(24), one, one, 1 << 20) == -1
+    assert b"16-byte aligned" in _lib.lib.lbt_last_error()
+    ws = _lib.lib.lbt_weighted_gradient_sums
+    assert ws(None, _lib.LBT_OBJ_SQUARED_ERROR, one, two, None, 1.0, 10, 1, C.c_void_p(1024), C.c_void_p(2048),
+              C.c_void_p(1024 + 16)) == -1
+    assert b"alias" in _lib.lib.lbt_last_error()
     with pytest.raises(_lib.LbtError):
         _lib.check(rc)
     # the stages of a level

@@ -276,7 +276,7 @@ def test_predict_matches_oracle_multi_tree_multi_output():
     assert np.array_equal(gu.cpu(ops.predict(X, [], 3)), np.zeros((30000, 3)))
 
 
-@pytest.mark.parametrize("f,k", [(13, 1), (100, 1), (200, 3), (330, 1)])
+@pytest.mark.parametrize("f,k", [(13, 1), (100, 1), (200, 3), (330, 1), (40, 11), (13, 17)])
 def test_predict_tiled_and_per_node_paths_agree_with_oracle(f, k):
     """Mixed tree sizes, feature counts that take 4, 8 or 16 lanes per row (one not a multiple of
     four), a row count that is not a multiple of the tile, thresholds that equal feature values or
@@ -315,7 +315,7 @@ def test_predict_tiled_and_per_node_paths_agree_with_oracle(f, k):
 
 
 @pytest.mark.parametrize("f,k,dtype", [(13, 1, np.float32), (100, 3, np.float32), (330, 1, np.float32),
-                                       (40, 2, np.float64)])
+                                       (40, 2, np.float64), (24, 19, np.float32), (9, 9, np.float64)])
 def test_packed_ensemble_predicts_like_the_oracle(f, k, dtype):
     import gpu_util as gu
     import oracle_lib as orc
