@@ -38,6 +38,8 @@ def parse():
                     help="bytes of histograms BuildTreeTask keeps (0 = the reference's 1e9, build_tree.cu:1004); a larger "
                          "cache builds the same trees and lets deeper levels derive siblings by subtraction")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default run only: leave out the short legs of configurations 3, 4 and 5 that follow the headline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 4 GiB device copy five times (to scale rocprofv3's FETCH_SIZE / "
                          "WRITE_SIZE counters against a kernel of known traffic)")
@@ -127,29 +129,34 @@ def measured_traffic(workload, rows, features):
     return out
 
 
-def bench_training(args):
+def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
+    """One training configuration. light: the timed rounds only (no second flow, no per-class
+    breakdown, no CPU baseline): the short legs that follow the headline in the default run."""
     import numpy as np
     import torch
 
     from lbtree import _lib, datasets, ops
 
-    cfg = args.config
+    cfg = args.config if cfg is None else cfg
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
     lr = 0.1
     n_classes = 0
+    rows_override = 0 if light else args.rows
     if cfg == 1:
         Xh, yh = datasets.config1()
         X, y = ops.as_device(Xh), ops.as_device(yh, torch.float64)
         depth, S, name = 6, 256, "cfg1"
     elif cfg == 2:
-        rows = args.rows or 10_000_000
+        rows = rows_override or 10_000_000
         X, y = datasets.config2(rows, 100)
         depth, S, name = 8, 256, "cfg2"
     elif cfg == 3:
-        rows = args.rows or 2_000_000
+        rows = rows_override or 2_000_000
         X, y = datasets.config3(rows, 200, 8)
         depth, S, name, n_classes = 8, 256, "cfg3", 8
     else:
-        rows = args.rows or 1_000_000
+        rows = rows_override or 1_000_000
         X, y = datasets.config4(rows, 50)
         depth, S, name = 12, 512, "cfg4"
     n, f = X.shape
@@ -199,7 +206,7 @@ def bench_training(args):
         return float(((pred[:, 0] - y) ** 2).mean())
 
     loss0 = loss()
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         one_round()
     torch.cuda.synchronize()
     # the timed rounds carry HIP events around the two histogram-stage kernels only (18 events
@@ -207,30 +214,34 @@ def bench_training(args):
     _lib.profile_reset()
     _lib.profile_enable(2)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         one_round()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     prof = _lib.profile_get()
     loss1 = loss()
     _lib.profile_reset()
-    _lib.profile_enable(1)
-    for _ in range(2):
-        one_round()
-    torch.cuda.synchronize()
-    _lib.profile_enable(0)
-    prof_all = _lib.profile_get()
-    # the other flow of a round, in the same run and on the same model: the reference loop's own
-    # steps (gradient as separate array operations, BuildTreeTask, PredictTask of the new tree)
-    # when the timed rounds took the fused steps, and the other way round
-    other_steps = max(2, min(args.steps, 5))
-    one_round(not args.reference_flow)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(other_steps):
+    prof_all = None
+    other_rate = None
+    other_steps = max(2, min(steps, 5))
+    if not light:
+        _lib.profile_enable(1)
+        for _ in range(2):
+            one_round()
+        torch.cuda.synchronize()
+        _lib.profile_enable(0)
+        prof_all = _lib.profile_get()
+        # the other flow of a round, in the same run and on the same model: the reference loop's own
+        # steps (gradient as separate array operations, BuildTreeTask, PredictTask of the new tree)
+        # when the timed rounds took the fused steps, and the other way round
         one_round(not args.reference_flow)
-    torch.cuda.synchronize()
-    other_rate = other_steps / (time.perf_counter() - t0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(other_steps):
+            one_round(not args.reference_flow)
+        torch.cuda.synchronize()
+        other_rate = other_steps / (time.perf_counter() - t0)
+    _lib.profile_enable(0)
 
     # The reference keeps 1e9 bytes of histograms (build_tree.cu:1004); a tree whose levels outgrow that
     # builds both children of every node from there on. With room for the whole tree (this GPU has 288 GB)
@@ -249,7 +260,6 @@ def bench_training(args):
     hist, binning = prof["histogram"], prof["binning"]
     elem = X.element_size()
     bin_bytes = 1 if S <= 256 else 2
-    steps = args.steps
 
     def gbps(byts, ms):
         return byts / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
@@ -279,12 +289,12 @@ def bench_training(args):
     out = {
         "metric": "boosting rounds/sec + histogram HBM GB/s (% peak), 10M×100 depth 8" if cfg == 2
         else "boosting rounds/sec + histogram HBM GB/s (%% peak), %s" % name,
-        "value": args.steps / dt,
+        "value": steps / dt,
         "unit": "rounds/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": dt / args.steps * 1e3,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": dt / steps * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -300,8 +310,12 @@ def bench_training(args):
             "prediction_update": "PredictTask" if args.reference_flow else "row->leaf map from BuildTreeTask",
             # a round as the reference loop runs it (legateboost.py:254-275): gradient arithmetic as
             # array operations, BuildTreeTask, PredictTask of the new tree; measured in this run
-            "reference_flow_rounds_per_s": args.steps / dt if args.reference_flow else other_rate,
-            "fused_flow_rounds_per_s": other_rate if args.reference_flow else args.steps / dt,
+            "reference_flow_rounds_per_s": steps / dt if args.reference_flow else other_rate,
+            "fused_flow_rounds_per_s": other_rate if args.reference_flow else steps / dt,
+            # the fractions below are averages over these boosting rounds (0-based) of one model: the rows a
+            # level has to build (the smaller child of every split) change from round to round, and with them
+            # the share of the fixed root level in a tree's histogram bytes
+            "rounds_timed": [warmup, warmup + steps - 1],
             "other_flow_steps": other_steps,
             "rounds_per_s_with_histograms_of_the_whole_tree_cached": whole_rate,
             "whole_tree_histogram_bytes": whole_tree,
@@ -345,9 +359,19 @@ def bench_training(args):
                 "achieved": gbps(stage_bytes, stage_ms), "frac": gbps(stage_bytes, stage_ms) / HBM_PEAK_GBS,
             },
         },
-        # two rounds after the timed ones, every kernel class bracketed by events
-        "kernel_ms_per_round": {c: prof_all[c]["ms"] / 2 for c in _lib.PROF_CLASSES},
     }
+    if light:
+        r = out["roofline"]
+        return {"workload": out["config"]["workload"], "value": out["value"], "unit": "rounds/s", "steps": steps,
+                "warmup": warmup, "ms_per_step": out["ms_per_step"],
+                "rounds_per_s_with_histograms_of_the_whole_tree_cached": whole_rate,
+                "roofline": {"kernel": r["kernel"], "frac": r["frac"], "avg_launch_ms": r["avg_launch_ms"],
+                             "frac_reference_accounting": r["frac_reference_accounting"],
+                             "stage_ms_per_tree": stage_ms / steps, "stage_GB_per_tree_reference_accounting": stage_bytes / steps / 1e9,
+                             "binning_ms": r["binning_kernel"]["avg_launch_ms"],
+                             "level_ms": [lv["ms"] for lv in levels]}}
+    # two rounds after the timed ones, every kernel class bracketed by events
+    out["kernel_ms_per_round"] = {c: prof_all[c]["ms"] / 2 for c in _lib.PROF_CLASSES}
     if not args.no_cpu_baseline:
         # config 2 (the headline) on all of its rows; the wider configurations on a row sample
         ns = n if cfg <= 2 else min(n, 500_000)
@@ -356,38 +380,46 @@ def bench_training(args):
     return out
 
 
-def bench_predict(args):
+def bench_predict(args, steps=None, warmup=None, light=False):
     import numpy as np
     import torch
 
     import cpu_variant_lib as cv
     from lbtree import _lib, datasets, ops
 
-    rows = args.rows or 20_000_000
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    rows = (0 if light else args.rows) or 20_000_000
     trees = datasets.config5_ensemble()
     X = datasets.config5_X(rows)
-    for _ in range(max(1, args.warmup)):
+    for _ in range(max(1, warmup)):
         ops.predict(X, trees, 1)
     torch.cuda.synchronize()
     _lib.profile_reset()
     _lib.profile_enable(True)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         out_t = ops.predict(X, trees, 1)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     _lib.profile_enable(False)
     byts = rows * (64 * 4 + 8)
-    achieved = byts * args.steps / dt / 1e9
+    achieved = byts * steps / dt / 1e9
+    if light:
+        return {"workload": "cfg5: PredictTask, 1000 trees of depth 8, X %dx64 f32, out f64" % rows,
+                "value": rows * steps / dt, "unit": "rows/s", "steps": steps, "warmup": max(1, warmup),
+                "ms_per_step": dt / steps * 1e3, "node_steps_per_s": rows * 8000 * steps / dt,
+                "roofline": {"kernel": "predict_tile_kernel", "bound": "hbm", "frac": achieved / HBM_PEAK_GBS,
+                             "limited_by": "lds"}}
     out = {
         "metric": "PredictTask rows/s, 1000 trees depth 8, 20M×64",
-        "value": rows * args.steps / dt,
+        "value": rows * steps / dt,
         "unit": "rows/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": dt / steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64", "data": "synthetic",
         "config": {"workload": "cfg5: PredictTask, 1000 trees of depth 8, X %dx64 f32, out f64" % rows,
-                   "rows": rows, "trees": 1000, "row_trees_per_s": rows * 1000 * args.steps / dt,
-                   "node_steps_per_s": rows * 8000 * args.steps / dt},
+                   "rows": rows, "trees": 1000, "row_trees_per_s": rows * 1000 * steps / dt,
+                   "node_steps_per_s": rows * 8000 * steps / dt},
         # X read once and the output written once are all the HBM bytes this path needs (achieved /
         # peak / frac price those); what bounds the kernel is the LDS: every node step of a wave
         # is two LDS reads (node, feature value), which the counters put at 8.2 cycles each
@@ -398,7 +430,7 @@ def bench_predict(args):
                      "limited_by": "lds",
                      "lds": {"wave_level_node_steps": rows * 8000 / 64,
                              "cycles_per_wave_level_node_step_and_cu":
-                                 dt / args.steps * 2.4e9 / (rows * 8000 / 64 / 256),
+                                 dt / steps * 2.4e9 / (rows * 8000 / 64 / 256),
                              "lds_reads_per_node_step": 2.1, "lds_cycles_per_read_measured": 8.2,
                              "clock_assumed_GHz": 2.4}},
     }
@@ -447,7 +479,34 @@ def main():
               % args.gpus, file=sys.stderr)
         sys.exit(2)
     out = bench_predict(args) if args.config == 5 else bench_training(args)
+    if args.config == 2 and not args.no_other_configs and not args.rows:
+        # the other benchmark configurations in the same run, a few rounds each, so that their
+        # rates are on record beside the headline's (each can also be run alone with --config)
+        out["other_configs"] = other_configs(args)
     print(json.dumps(out))
+
+
+def _release_device_memory():
+    import gc
+
+    import torch
+
+    from lbtree import ops
+
+    ops._workspace.clear()
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def other_configs(args):
+    legs = {}
+    _release_device_memory()
+    for cfg in (3, 4):
+        legs["cfg%d" % cfg] = bench_training(args, cfg=cfg, steps=5, warmup=2, light=True)
+        _release_device_memory()
+    legs["cfg5"] = bench_predict(args, steps=2, warmup=1, light=True)
+    _release_device_memory()
+    return legs
 
 
 if __name__ == "__main__":
