@@ -38,6 +38,10 @@ def parse():
                     help="bytes of histograms BuildTreeTask keeps (0 = the reference's 1e9, build_tree.cu:1004); a larger "
                          "cache builds the same trees and lets deeper levels derive siblings by subtraction")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--only-timed", action="store_true",
+                    help="run the warm-up and the timed rounds only (no per-class breakdown rounds, no rounds in the other "
+                         "flow, no CPU baseline, no other configurations): what a profiler run wants, every launch of "
+                         "the process then belongs to the rounds the printed figures describe")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="default run only: leave out the short legs of configurations 3, 4 and 5 that follow the headline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -126,12 +130,18 @@ def measured_traffic(workload, rows, features):
         if (kv.get("workload") == workload and int(kv.get("rows", -1)) == rows
                 and int(kv.get("features", -1)) == features and kv.get("source") == tag):
             out[parts[0]] = float(kv["traffic_bytes_per_launch"])
+            if "algorithmic_bytes_per_launch" in kv:
+                # the algorithmic bytes of the very launches the counters were read on
+                out[parts[0] + ":ratio"] = float(kv["traffic_bytes_per_launch"]) / float(kv["algorithmic_bytes_per_launch"])
     return out
 
 
 def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
-    """One training configuration. light: the timed rounds only (no second flow, no per-class
-    breakdown, no CPU baseline): the short legs that follow the headline in the default run."""
+    """One training configuration. light: a short leg that follows the headline in the default run:
+    the timed rounds only (no second flow, no per-class breakdown, no CPU baseline) and a compact
+    result. args.only_timed runs the same rounds and returns the full result."""
+    compact = light
+    light = light or args.only_timed
     import numpy as np
     import torch
 
@@ -248,7 +258,7 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
     # the same trees come out and every level derives siblings by subtraction: measured in the same run.
     whole_tree = (2 ** depth - 1) * k * f * S * 16
     whole_rate = None
-    if whole_tree > (args.hist_cache_bytes or 1000000000):
+    if whole_tree > (args.hist_cache_bytes or 1000000000) and not args.only_timed:
         one_round(cache=whole_tree)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -284,6 +294,9 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
                        "GB_cached_bins": lv["bytes"] / steps / 1e9, "GBps_cached_bins": gbps(lv["bytes"], lv["ms"]),
                        "GB_reference_accounting": ref_bytes / steps / 1e9})
     stage_ms = hist["ms"] + binning["ms"]
+    # the root launch's own-format bytes include the feature-major copy of the bins it writes for the
+    # position updates; the histogram itself does not need it
+    copy_bytes = n * f * bin_bytes * steps if depth >= 2 else 0.0
     traffic = measured_traffic(name, n, f)
     hist_achieved = gbps(hist["bytes"], hist["ms"])
     out = {
@@ -328,7 +341,10 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": hist_achieved / HBM_PEAK_GBS,
+            "frac_without_feature_major_copy": gbps(hist["bytes"] - copy_bytes, hist["ms"]) / HBM_PEAK_GBS,
             "traffic": traffic.get("binned_histogram_kernel"),
+            # measured HBM bytes over algorithmic bytes, both of the profiled run's own launches
+            "traffic_over_algorithmic": traffic.get("binned_histogram_kernel:ratio"),
             "traffic_source": "profiles/hbm_traffic_%s.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE), applies when its "
                               "source tag equals %s" % (name, source_tag()),
             # the histogram stage of a tree (binning pass + every histogram launch) against the bytes
@@ -350,6 +366,7 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
                 "achieved": gbps(binning["bytes"], binning["ms"]),
                 "frac": gbps(binning["bytes"], binning["ms"]) / HBM_PEAK_GBS,
                 "traffic": traffic.get("bin_rows_kernel"),
+                "traffic_over_algorithmic": traffic.get("bin_rows_kernel:ratio"),
             },
             # the whole histogram stage of a tree (both kernels) against the bytes the
             # reference's histogram kernel would have to move for the same levels
@@ -360,7 +377,7 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
             },
         },
     }
-    if light:
+    if compact:
         r = out["roofline"]
         return {"workload": out["config"]["workload"], "value": out["value"], "unit": "rounds/s", "steps": steps,
                 "warmup": warmup, "ms_per_step": out["ms_per_step"],
@@ -370,6 +387,8 @@ def bench_training(args, cfg=None, steps=None, warmup=None, light=False):
                              "stage_ms_per_tree": stage_ms / steps, "stage_GB_per_tree_reference_accounting": stage_bytes / steps / 1e9,
                              "binning_ms": r["binning_kernel"]["avg_launch_ms"],
                              "level_ms": [lv["ms"] for lv in levels]}}
+    if light:
+        return out
     # two rounds after the timed ones, every kernel class bracketed by events
     out["kernel_ms_per_round"] = {c: prof_all[c]["ms"] / 2 for c in _lib.PROF_CLASSES}
     if not args.no_cpu_baseline:
@@ -434,7 +453,7 @@ def bench_predict(args, steps=None, warmup=None, light=False):
                              "lds_reads_per_node_step": 2.1, "lds_cycles_per_read_measured": 8.2,
                              "clock_assumed_GHz": 2.4}},
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.only_timed:
         cores = max(1, min(16, os.cpu_count() or 1))
         ns = 20000
         Xs = X[:ns].cpu().numpy()
@@ -479,7 +498,7 @@ def main():
               % args.gpus, file=sys.stderr)
         sys.exit(2)
     out = bench_predict(args) if args.config == 5 else bench_training(args)
-    if args.config == 2 and not args.no_other_configs and not args.rows:
+    if args.config == 2 and not args.no_other_configs and not args.rows and not args.only_timed:
         # the other benchmark configurations in the same run, a few rounds each, so that their
         # rates are on record beside the headline's (each can also be run alone with --config)
         out["other_configs"] = other_configs(args)

@@ -1187,6 +1187,8 @@ struct BinnedArgs {
   const int32_t* groups;
   HistView hist;
   Stripes stripes;  // layout of the LDS sub-histogram
+  int lanes;        // lanes per row for every group of the launch; 0: as many as the group's own features need
+  int sync_every;   // tiles between two meeting points of the root launch's workgroups
 };
 
 // The 16 bytes of `w` rotated down by t bytes: byte v of the result is byte (v + t) mod 16 of w.
@@ -1260,7 +1262,12 @@ __global__ void __launch_bounds__(kHistThreads)
   }
 
   const RecInfo ri        = a.rec[group];
-  const int lanes_per_row = (gs + BV - 1) / BV;
+  // With the same number of lanes per row in every group (a narrower group's last lanes then add the
+  // zero bytes of its record's padding to columns that nothing reads) the workgroups of the groups
+  // that walk the same rows run the same instructions tile after tile and stay side by side
+  // without waiting for each other: the cache line that holds a row's records is then still in the
+  // L2 when the second of them asks for it.
+  const int lanes_per_row = a.lanes > 0 ? a.lanes : (gs + BV - 1) / BV;
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
   const bool active       = rsub < w.rpp;
@@ -1360,9 +1367,9 @@ __global__ void __launch_bounds__(kHistThreads)
       // of them fetched is still in the L2 when the next one asks for it. Only a hint: after
       // kPairSyncSpins polls a workgroup goes on regardless.
       const int done = tile - t_begin;
-      if (pair_sync != nullptr && done > 0 && done % kPairSyncTiles == 0) {
+      if (pair_sync != nullptr && done > 0 && done % a.sync_every == 0) {
         if (threadIdx.x == 0) {
-          const int want = done / kPairSyncTiles * w.n_gk;
+          const int want = done / a.sync_every * w.n_gk;
           __hip_atomic_fetch_add(pair_sync + chunk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           for (int spin = 0; spin < kPairSyncSpins; spin++) {
             if (__hip_atomic_load(pair_sync + chunk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= want) break;
@@ -1578,7 +1585,7 @@ int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& 
     // single-output trees, whose root launch is bound by the memory traffic the meetings save; with
     // several outputs the records are found in the L2 anyway (the workgroups of the other outputs
     // asked for them) and the waiting is all that is left (2M x 200, 8 outputs: 1.27 ms with, 0.95 ms without)
-    kRoot && a.K == 1 && a.w.n_gk > 1 && a.w.all_resident && a.w.n_chunks <= kPairSyncSlots ? hs.pair_sync : nullptr,
+    kRoot && a.K == 1 && a.w.n_gk > 1 && a.w.all_resident && a.w.n_chunks <= kPairSyncSlots && a.sync_every > 0 ? hs.pair_sync : nullptr,
     sink);
   return LBT_OK;
 }
@@ -1702,6 +1709,8 @@ int hist_launch_t(hipStream_t stream, const HistSetup& hs, const HistBatch& b, i
     a.groups       = hs.groups;
     a.hist         = b.hist;
     a.stripes      = Stripes{hs.stripe_log, hs.stripe_bins};
+    a.lanes        = hs.even_lanes;
+    a.sync_every   = kPairSyncTiles;
     PartialSink sink{hs.partials, hs.partial_lists, hs.partial_list_count, hs.partial_count, 0, hs.partial_stride};
     if (hs.partials != nullptr && static_cast<int64_t>(w.n_nodes) * w.n_gk <= kPartialMaxLists)
       sink.slots = hs.partial_slots;
@@ -2056,6 +2065,18 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       pitch += ri.size;
     }
     hs.max_rec_stride = pitch;
+    // the same lanes per row for all groups (see binned_histogram_kernel): when the striped layout is
+    // used, the records carry the gradient pair (one output: the groups' workgroups are bound by the
+    // memory traffic they can share) and every record is long enough for the widest group's lanes
+    hs.even_lanes = 0;
+    if (hs.stripe_log >= 0 && hs.embed && hs.n_groups > 1) {
+      int lanes = 0;
+      for (int g = 0; g < hs.n_groups; g++) lanes = std::max(lanes, (groups[g + 1] - groups[g] + hs.bvec - 1) / hs.bvec);
+      bool fits = true;
+      for (int g = 0; g < hs.n_groups; g++) fits = fits && lanes * chunk <= rec[g].size;
+      fits = fits && lanes * hs.bvec <= (1 << hs.stripe_log);
+      if (fits) hs.even_lanes = lanes;
+    }
     for (int g = 0; g < hs.n_groups; g++) {
       RecInfo& ri = rec[g];
       ri.stride   = pitch;
