@@ -1294,6 +1294,22 @@ __global__ void __launch_bounds__(kHistThreads)
       c_base[v] = fl + v < gs ? a.row_pointers[f0 + fl + v] - bin0 : nb + threadIdx.x;
     }
   }
+  // The bytes of a lane's 16 that lie past the group's last feature are zeros (record padding, the
+  // blanked gradient pair): added as they are, they would all fall into bin 0 of their column, and
+  // the lanes that hold the same column in the four quarters of a wave (thread t, t + 16, ...)
+  // would hit one address at every step, which the LDS serialises (3 cycles of
+  // SQ_LDS_ADDR_CONFLICT per atomic, one more cycle per wave-level atomic in a kernel that does
+  // nothing else; 1 % of these launches, where the LDS is busy less than half of the time). Each
+  // quarter sends them to a bin of its own instead; nothing reads those columns.
+  uint4 pad_or = make_uint4(0u, 0u, 0u, 0u);
+  if constexpr (kStriped) {
+    const uint32_t q4 = min((static_cast<uint32_t>(threadIdx.x) >> 4) & 3u, static_cast<uint32_t>(max(st.bins, 1) - 1));
+    uint32_t pw[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+      if (fl + j >= gs) pw[j >> 2] |= q4 << (8 * (j & 3));
+    pad_or = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+  }
   const int stripe_shift = st.log_w + 3;  // a bin's row of the striped array, in bytes
   const unsigned long long max_abs = qstats[0];
   const int n_tiles = meta->n_tiles;
@@ -1460,7 +1476,13 @@ __global__ void __launch_bounds__(kHistThreads)
     if constexpr (kStriped) {
       // from here on a lane's bins stand in its own order (the feature-major copy above took them as loaded)
 #pragma unroll
-      for (int u = 0; u < kRows; u++) b_c[u] = rotate_bytes(b_c[u], rot);
+      for (int u = 0; u < kRows; u++) {
+        b_c[u].x |= pad_or.x;
+        b_c[u].y |= pad_or.y;
+        b_c[u].z |= pad_or.z;
+        b_c[u].w |= pad_or.w;
+        b_c[u] = rotate_bytes(b_c[u], rot);
+      }
     }
     if (!direct) {
 #pragma unroll
