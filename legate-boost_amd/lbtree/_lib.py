@@ -2,12 +2,17 @@
 
 The library is the only compute path: if it has not been built the import
 fails, there is no fallback.
+
+Environment: LBTREE_SO, when set and not empty, is the path of the shared
+library to load instead of csrc/liblbtree.so beside this package (to compare
+two builds of the kernels from one checkout). It has to export the same
+symbols (binding them below raises otherwise) and to exist; nothing else is
+tried.
 """
 import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# LBTREE_SO selects another build of the same library (kernel tuning)
 SO_PATH = os.environ.get("LBTREE_SO") or os.path.join(os.path.dirname(_HERE), "csrc", "liblbtree.so")
 
 LBT_OK = 0
