@@ -1202,6 +1202,13 @@ __device__ __forceinline__ uint4 rotate_bytes(const uint4& w, int t)
                     __builtin_amdgcn_alignbyte(w2, z2, b), __builtin_amdgcn_alignbyte(x2, w2, b));
 }
 
+// The value that lane kLane of the caller's aligned group of four lanes holds (all four have to be active).
+template <int kLane>
+__device__ __forceinline__ int quad_lane(int v)
+{
+  return __builtin_amdgcn_update_dpp(0, v, kLane * 0x55, 0xf, 0xf, false);
+}
+
 // 4 x 4 byte transpose: input word r is row r and its byte b is feature b; output word b holds
 // feature b of rows 0..3.
 __device__ __forceinline__ void turn_bytes(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t (&out)[4])
@@ -1224,15 +1231,22 @@ __device__ __forceinline__ void turn_bytes(uint32_t w0, uint32_t w1, uint32_t w2
 // costs no second pass over the cache.
 // kStriped (one-byte bins): the LDS sub-histogram is striped (see Stripes) and every lane takes the
 // 16 bins of a row in its own rotated order.
+// kQuad (striped, kEmbed): every group of the launch has four lanes per row (and a lane four rows per
+// tile), so the lanes of a row are an aligned group of four, and what all of them need one of them loads
+// and hands round with a cross-lane move: a vector memory instruction costs by the cache lines it
+// touches and holds registers until it returns, the move is one vector instruction. Below the root lane
+// u of the four loads the position of the tile's row u. The record is the four lanes' 64 bytes and its
+// last 8 the gradient pair: the pair comes out of the fourth lane's bins.
 constexpr int kStripeMaxW = 256;  // widest group the striped layout serves, in features
 
-template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped>
+template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped, bool kQuad>
 __global__ void __launch_bounds__(kHistThreads)
   binned_histogram_kernel(BinnedArgs a, LBT_WALK_PARAMS, const unsigned char* __restrict__ cache,
                           const int2* __restrict__ qgh, BinT* __restrict__ bins_t, int64_t bins_t_stride,
                           int32_t* pair_sync, PartialSink sink)
 {
   static_assert(!kStriped || BV == 16, "the striped layout is built for lanes that hold 16 one-byte bins");
+  static_assert(!kQuad || (kStriped && kEmbed), "four lanes per 64-byte record: a mode of the striped kernel");
   __shared__ int s_slot;
   __shared__ int s_off[kStriped ? kStripeMaxW : 1];  // striped: first bin of every feature in the group's run of bins
   using Word = typename BinVec<BinT, BV>::type;
@@ -1267,7 +1281,7 @@ __global__ void __launch_bounds__(kHistThreads)
   // that walk the same rows run the same instructions tile after tile and stay side by side
   // without waiting for each other: the cache line that holds a row's records is then still in the
   // L2 when the second of them asks for it.
-  const int lanes_per_row = a.lanes > 0 ? a.lanes : (gs + BV - 1) / BV;
+  const int lanes_per_row = kQuad ? 4 : (a.lanes > 0 ? a.lanes : (gs + BV - 1) / BV);
   const int lr            = threadIdx.x % lanes_per_row;
   const int rsub          = threadIdx.x / lanes_per_row;
   const bool active       = rsub < w.rpp;
@@ -1328,8 +1342,17 @@ __global__ void __launch_bounds__(kHistThreads)
   const bool owners = static_cast<unsigned long long>(w.tile_rows) * max_abs <= 2147483647ULL;
   __syncthreads();
 
-  auto load_rows = [&](const Tile& t, int (&row)[kRows]) -> unsigned {
+  // positions a lane keeps per tile: with kQuad only that of the row with its own number among the four lanes
+  constexpr int kPos = kQuad && !kRoot ? 1 : kRows;
+  auto load_rows = [&](const Tile& t, int (&row)[kPos]) -> unsigned {
     unsigned valid = 0;
+    if constexpr (kQuad && !kRoot) {
+      const int mine = t.r0 + rsub + lr * w.rpp;
+      row[0]         = positions[mine < t.r1 ? mine : t.r0];
+#pragma unroll
+      for (int u = 0; u < kRows; u++) valid |= t.r0 + rsub + u * w.rpp < t.r1 ? (1u << u) : 0u;
+      return valid;
+    }
 #pragma unroll
     for (int u = 0; u < kRows; u++) {
       const int rr  = kRoot ? t.r0 + kRows * rsub + u : t.r0 + rsub + u * w.rpp;
@@ -1342,16 +1365,30 @@ __global__ void __launch_bounds__(kHistThreads)
     }
     return valid;
   };
-  auto load_data = [&](const int (&row)[kRows], Word (&bw)[kRows], int2 (&q)[kRows]) {
+  // gradient pairs a lane loads per tile: none (one unused slot) when they come out of the fourth lane's bins
+  constexpr int kPairs = kQuad ? 1 : kRows;
+  auto load_data = [&](const int (&row)[kPos], Word (&bw)[kRows], int2 (&q)[kPairs]) {
+    int rws[kRows];
+    if constexpr (kQuad && !kRoot) {
+      rws[0] = quad_lane<0>(row[0]);
+      rws[1] = quad_lane<1>(row[0]);
+      rws[2] = quad_lane<2>(row[0]);
+      rws[3] = quad_lane<3>(row[0]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kRows; u++) rws[u] = row[u];
+    }
 #pragma unroll
     for (int u = 0; u < kRows; u++) {
-      const int64_t rw          = row[u];
+      const int64_t rw          = rws[u];
       const unsigned char* recp = my_rec + rw * stride;
       bw[u]                     = *reinterpret_cast<const Word*>(recp + my_off);
-      if constexpr (kEmbed)
+      if constexpr (kQuad) {
+      } else if constexpr (kEmbed) {
         q[u] = *reinterpret_cast<const int2*>(recp + ri.q_off);
-      else
+      } else {
         q[u] = qgh[rw * a.K + k];
+      }
     }
   };
 
@@ -1359,12 +1396,14 @@ __global__ void __launch_bounds__(kHistThreads)
   TileWindow win{s_tile_window, tiles, 0, t_end};
   win.fill(t_begin);
   Tile tc{}, tn{}, tnn{};
-  int row_c[kRows], row_n[kRows], row_nn[kRows];
+  int row_c[kPos], row_n[kPos], row_nn[kPos];
   Word b_c[kRows], b_n[kRows];
-  int2 q_c[kRows], q_n[kRows];
+  int2 q_c[kPairs], q_n[kPairs];
   unsigned valid_c = 0, valid_n = 0, valid_nn = 0;
 #pragma unroll
-  for (int u = 0; u < kRows; u++) row_c[u] = row_n[u] = row_nn[u] = 0;
+  for (int u = 0; u < kPos; u++) row_c[u] = row_n[u] = row_nn[u] = 0;
+#pragma unroll
+  for (int u = 0; u < kPairs; u++) q_c[u] = q_n[u] = make_int2(0, 0);
   if (t_begin < t_end) {
     tc      = win.get(t_begin);
     valid_c = load_rows(tc, row_c);
@@ -1422,6 +1461,14 @@ __global__ void __launch_bounds__(kHistThreads)
       }
       acc += nrows;
       node_rows += nrows;
+    }
+    int2 qv[kRows];
+#pragma unroll
+    for (int u = 0; u < kRows; u++) {
+      if constexpr (kQuad)
+        qv[u] = make_int2(quad_lane<3>(static_cast<int>(b_c[u].z)), quad_lane<3>(static_cast<int>(b_c[u].w)));
+      else
+        qv[u] = q_c[u];
     }
     if constexpr (kEmbed && BV == 16) {
 #pragma unroll
@@ -1488,7 +1535,7 @@ __global__ void __launch_bounds__(kHistThreads)
 #pragma unroll
       for (int u = 0; u < kRows; u++) {
         if (valid_c & (1u << u)) {
-          const unsigned long long packed = pack_pair(q_c[u].x, q_c[u].y);
+          const unsigned long long packed = pack_pair(qv[u].x, qv[u].y);
           int rel[BV];
           unpack_bins<BinT, BV>(b_c[u], rel);
 #pragma unroll
@@ -1525,8 +1572,8 @@ __global__ void __launch_bounds__(kHistThreads)
               bin  = c_base[v] + rel[v];
             }
             if (mine) {
-              atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(q_c[u].x));
-              atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(q_c[u].y));
+              atomic_add_i64(&gdst[bin].grad, static_cast<int64_t>(qv[u].x));
+              atomic_add_i64(&gdst[bin].hess, static_cast<int64_t>(qv[u].y));
             }
           }
         }
@@ -1537,12 +1584,14 @@ __global__ void __launch_bounds__(kHistThreads)
     valid_c = valid_n;
     valid_n = valid_nn;
 #pragma unroll
-    for (int u = 0; u < kRows; u++) {
+    for (int u = 0; u < kPos; u++) {
       row_c[u] = row_n[u];
       row_n[u] = row_nn[u];
-      b_c[u]   = b_n[u];
-      q_c[u]   = q_n[u];
     }
+#pragma unroll
+    for (int u = 0; u < kRows; u++) b_c[u] = b_n[u];
+#pragma unroll
+    for (int u = 0; u < kPairs; u++) q_c[u] = q_n[u];
   }
   __syncthreads();
   if (cur_node >= 0)
@@ -1591,15 +1640,15 @@ int launch_bin_rows_t(hipStream_t stream, const HistSetup& hs, const BinRowsArgs
   return launch_bin_rows<T, VEC, uint16_t, false>(stream, hs, a, b, grid);
 }
 
-template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped>
+template <typename BinT, int BV, bool kEmbed, bool kRoot, bool kStriped, bool kQuad = false>
 int launch_binned_as(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, const HistBatch& b, unsigned grid,
                      const PartialSink& sink)
 {
   static std::atomic<bool> attr_set[kMaxDevices] = {};
   // the striped kernel keeps a table of feature offsets in static LDS and never asks for more than this
-  LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped>,
+  LBT_TRY(allow_dynamic_lds(binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped, kQuad>,
                             kStriped ? kLdsBudget - 8 * 1024 : kLdsBudget, attr_set));
-  binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
+  binned_histogram_kernel<BinT, BV, kEmbed, kRoot, kStriped, kQuad><<<grid, kHistThreads, hs.blds_bytes, stream>>>(
     a, b.rows, hs.tiles, hs.meta, b.qstats, static_cast<const unsigned char*>(hs.binned), b.qgh,
     static_cast<BinT*>(hs.bins_t), hs.bins_t_stride,
     // meeting points only between workgroups that run at the same time: one that waits for a
@@ -1617,6 +1666,12 @@ int launch_binned(hipStream_t stream, const HistSetup& hs, const BinnedArgs& a, 
 {
   if constexpr (BV == 16) {
     if (a.stripes.log_w >= 0) {
+      if constexpr (kEmbed) {
+        if (hs.quad) {
+          if (root) return launch_binned_as<BinT, BV, kEmbed, true, true, true>(stream, hs, a, b, grid, sink);
+          return launch_binned_as<BinT, BV, kEmbed, false, true, true>(stream, hs, a, b, grid, sink);
+        }
+      }
       if (root) return launch_binned_as<BinT, BV, kEmbed, true, true>(stream, hs, a, b, grid, sink);
       return launch_binned_as<BinT, BV, kEmbed, false, true>(stream, hs, a, b, grid, sink);
     }
@@ -2098,6 +2153,14 @@ int hist_prepare(hipStream_t stream, HistSetup& hs, bool is_f64, int F, int K, i
       for (int g = 0; g < hs.n_groups; g++) fits = fits && lanes * chunk <= rec[g].size;
       fits = fits && lanes * hs.bvec <= (1 << hs.stripe_log);
       if (fits) hs.even_lanes = lanes;
+    }
+    // the kernel's mode for four lanes per row (see binned_histogram_kernel): single-output trees whose
+    // groups all have four lanes per row, by their own width or by even_lanes, and records of those lanes'
+    // 64 bytes with the pair in the last 8 (with several outputs the mode saves no load and was no faster)
+    hs.quad = hs.stripe_log >= 0 && hs.embed && kBinnedUnroll / 2 == 4;
+    for (int g = 0; g < hs.n_groups && hs.quad; g++) {
+      const int lanes = hs.even_lanes > 0 ? hs.even_lanes : (groups[g + 1] - groups[g] + hs.bvec - 1) / hs.bvec;
+      hs.quad         = lanes == 4 && rec[g].size == 64 && rec[g].q_off == 56;
     }
     for (int g = 0; g < hs.n_groups; g++) {
       RecInfo& ri = rec[g];

@@ -372,6 +372,7 @@ struct HistSetup {
   int stripe_log       = -1;       // log2 of the striped layout's row width in features; negative: [feature][bin]
   int stripe_bins      = 0;        // bins of the widest feature (rows of the striped array)
   int even_lanes       = 0;        // lanes per row shared by all groups of a histogram launch; 0: per group
+  bool quad            = false;    // single-output trees, four lanes per 64-byte record in every group: the histogram kernel's kQuad mode
   RecInfo* rec         = nullptr;  // [n_groups]
   int64_t max_rec_stride = 0;      // widest record, bytes
   int64_t* bin_base    = nullptr;  // [n_features] element offset of the feature's bin of row 0
