@@ -128,7 +128,7 @@ T* dense_out(legate::PhysicalStore store)
   // every node once a level outgrows that. The sums are integers, so any budget gives the same tree;
   // with room for the histograms of every level (levels 0 .. max_depth - 1, every bin distinct)
   // all levels derive one child of each pair by subtraction. Taken when a tenth of the free
-  // framebuffer holds it (2M x 200 with 8 outputs at depth 8: 1.7 GB, 132 -> 147 rounds per second),
+  // framebuffer holds it (2M x 200 with 8 outputs at depth 8: 1.7 GB, 132 -> 146 rounds per second),
   // else the reference's constant (0).
   p.hist_cache_bytes = 0;
   {
