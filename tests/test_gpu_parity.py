@@ -39,6 +39,8 @@ def _problem(seed, n, f, k, dtype=np.float32, lowcard=True):
     (3000, 11, 1, 3, 400, np.float32),    # ... with two-byte bins
     (2000, 200, 8, 3, 256, np.float32),   # 3 groups x 8 outputs would leave CUs idle: a fourth group is taken
     (2000, 300, 5, 3, 256, np.float32),
+    (20000, 100, 1, 9, 64, np.float32),   # four lanes per 64-byte record in two groups (52 + 48 features), down to
+    (3000, 52, 1, 6, 32, np.float32),     # nodes of a few rows, whose sums go to the histogram directly
 ])
 def test_build_tree_bit_exact(n, f, k, depth, s, dtype):
     import gpu_util as gu
