@@ -71,7 +71,10 @@ class LogLossObjective:
 
 class LBBase:
     def __init__(self, n_estimators=100, objective=None, base_models=(Tree(max_depth=8),), init="average",
-                 learning_rate=0.1, random_state=None, verbose=0):
+                 learning_rate=0.1, subsample=1.0, random_state=None, verbose=0):
+        if not 0.0 < subsample <= 1.0:
+            raise ValueError("subsample should be in (0, 1]")
+        self.subsample = subsample
         self.n_estimators = n_estimators
         self.objective = objective
         self.base_models = base_models
@@ -100,10 +103,22 @@ class LBBase:
     def _get_weighted_gradient(self, y, pred, sample_weight, learning_rate):
         fused = getattr(self._objective_instance, "fused", None)
         if fused is not None and pred.is_cuda:
-            return ops.weighted_gradient(fused, y, pred, sample_weight, learning_rate)
-        g, h = self._objective_instance.gradient(y, self._objective_instance.transform(pred))
-        g = g * sample_weight[:, None] * learning_rate
-        h = torch.clamp(h * sample_weight[:, None], min=1e-8)
+            g, h = ops.weighted_gradient(fused, y, pred, sample_weight, learning_rate)
+        else:
+            g, h = self._objective_instance.gradient(y, self._objective_instance.transform(pred))
+            g = g * sample_weight[:, None] * learning_rate
+            h = torch.clamp(h * sample_weight[:, None], min=1e-8)
+        if self.subsample < 1.0:
+            # legateboost.py:215-222: one Bernoulli(subsample) draw per row zeroes its gradient and hessian. The
+            # seed is taken from the estimator's RandomState at the same place as in the reference, so the tree
+            # seeds that follow are the reference's; the draws themselves come from torch's generator, not
+            # from cupynumeric's XORWOW stream, so which rows are kept is not comparable with the reference.
+            seed = int(self.random_state_.randint(0, 2**32, dtype=np.int64))
+            gen = torch.Generator(device=g.device).manual_seed(seed)
+            mask = (torch.rand(y.shape[0], generator=gen, device=g.device, dtype=torch.float64) < self.subsample)
+            mask = mask.to(torch.float64)[:, None]
+            g = g * mask
+            h = h * mask
         return g, h
 
     def _predict(self, X):

@@ -186,6 +186,40 @@ def test_regressor_and_update():
     assert np.allclose(_np(m.predict(X)), pred, rtol=1e-4, atol=1e-4)
 
 
+def test_subsample():
+    """test_estimator.py:191-227: on data that a deep tree overfits, keeping half of the rows per round
+    gives the lower test error (averaged over five data sets); and the seed of the row draw is taken from
+    the estimator's RandomState where the reference takes it, so the tree seeds are the reference's."""
+    import lbtree as lb
+    from sklearn.datasets import make_regression
+    from sklearn.model_selection import train_test_split
+
+    sub_mse, full_mse = [], []
+    for i in range(5):
+        X, y = make_regression(n_samples=1000, n_features=10, noise=10.0, random_state=i)
+        X_train, X_test, y_train, y_test = train_test_split(X, y, test_size=0.5, random_state=i)
+        params = dict(n_estimators=20, random_state=i, learning_rate=0.5,
+                      base_models=(lb.models.Tree(max_depth=12, alpha=0.0),))
+        sub = lb.LBRegressor(**params, subsample=0.5).fit(X_train, y_train)
+        full = lb.LBRegressor(**params).fit(X_train, y_train)
+        sub_mse.append(((_np(sub.predict(X_test)).ravel() - y_test) ** 2).mean())
+        full_mse.append(((_np(full.predict(X_test)).ravel() - y_test) ** 2).mean())
+    assert np.mean(sub_mse) < np.mean(full_mse)
+
+    # order of the draws from the estimator's RandomState: row-draw seed, then the tree's seed, every round
+    m = lb.LBRegressor(n_estimators=3, random_state=11, subsample=0.5, base_models=(lb.models.Tree(max_depth=2),))
+    rs = np.random.RandomState(7)
+    X = rs.random_sample((500, 4)).astype(np.float32)
+    m.fit(X, X[:, 0] + rs.normal(0, 0.1, 500))
+    expect = np.random.RandomState(11)
+    for _ in m:
+        expect.randint(0, 2**32, dtype=np.int64)
+        expect.randint(0, 2**31)
+    assert m.random_state_.randint(0, 2**31) == expect.randint(0, 2**31)
+    with pytest.raises(ValueError):
+        lb.LBRegressor(subsample=0.0)
+
+
 @pytest.mark.parametrize("num_class", [2, 5])
 def test_classifier(num_class):
     import lbtree as lb
